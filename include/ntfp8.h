@@ -1,0 +1,118 @@
+/* ntfp8 — C ABI of the MI355X (gfx950) FP8 linear hot path.
+ *
+ * This is the native plug-in point that stands where nanotron's `nanotron.fp8` package
+ * calls NVIDIA Transformer Engine's pybind module (`transformer_engine_extensions as tex`).
+ * Each entry point names the reference call it replaces (paths relative to the reference
+ * checkout).
+ *
+ * Conventions
+ *   - every data pointer is a DEVICE pointer owned by the caller (a torch tensor kept alive
+ *     on the Python side); the library never allocates, frees or synchronises;
+ *   - amax / scale / history values live in device memory: no host round trip;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *   - return value: 0 on success, a negative NTFP8_ERR_* code otherwise; argument errors are
+ *     detected on the host before anything is launched, so a bad call never faults the GPU;
+ *   - 2-D operands are row-major and contiguous; fp8 bytes are OCP e4m3fn / e5m2;
+ *   - `workspace` is NTFP8_WORKSPACE_BYTES of device memory that must be zero before its first
+ *     use; kernels leave it zero again, so it can be reused by stream-ordered calls.  Calls
+ *     that may overlap (different streams) need distinct workspaces.
+ */
+#ifndef NTFP8_H
+#define NTFP8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NTFP8_VERSION 1
+#define NTFP8_WORKSPACE_BYTES 64
+
+/* FP8 storage formats.  Reference: DTypes.FP8E4M3 / DTypes.FP8E5M2 (src/nanotron/fp8/dtypes.py:4-7),
+ * mapped to tex.DType.kFloat8E4M3 / kFloat8E5M2 at src/nanotron/fp8/tensor.py:39-55. */
+enum { NTFP8_E4M3 = 0, NTFP8_E5M2 = 1 };
+
+/* High-precision element types (tex.DType.kFloat32 / kFloat16 / kBFloat16, tensor.py:43-47). */
+enum { NTFP8_F32 = 0, NTFP8_F16 = 1, NTFP8_BF16 = 2 };
+
+enum {
+    NTFP8_OK = 0,
+    NTFP8_ERR_NULL = -1,        /* a required pointer is NULL */
+    NTFP8_ERR_ENUM = -2,        /* unknown format / dtype value */
+    NTFP8_ERR_SIZE = -3,        /* negative, zero or overflowing size */
+    NTFP8_ERR_ALIGN = -4,       /* pointer not aligned to its element type */
+    NTFP8_ERR_UNSUPPORTED = -5, /* valid request the library does not implement */
+    NTFP8_ERR_LAUNCH = -6,      /* HIP reported an error at launch */
+    NTFP8_ERR_ALIAS = -7        /* output overlaps an input */
+};
+
+int ntfp8_version(void);
+const char* ntfp8_strerror(int code);
+
+/* amax = max|x| (NaN-propagating) and the power-of-two scale derived from it.
+ * Replaces `tensor.abs().max()` + `update_scaling_factor(amax, 1.0, dtype)`
+ * (src/nanotron/fp8/tensor.py:25-26, 94-103), one launch instead of ~10.
+ * old_scale may be NULL (= INITIAL_SCALING_FACTOR 1.0, src/nanotron/fp8/constants.py:8). */
+int ntfp8_amax_scale(const void* x, int x_dtype, int64_t n, int fmt, int margin,
+                     const float* old_scale, float* amax_out, float* scale_out,
+                     void* workspace, void* stream);
+
+/* Element-wise update_scaling_factor on device arrays of n amax values
+ * (src/nanotron/fp8/tensor.py:77-105).  old_scale / out have n elements. */
+int ntfp8_update_scaling_factor(const float* amax, const float* old_scale, int fmt, int margin,
+                                float* out, int64_t n, void* stream);
+
+/* The same function for one host value (no GPU involved): what the reference evaluates on CPU
+ * tensors in FP8Linear.__init__ (src/nanotron/fp8/linear.py:33-42). */
+float ntfp8_update_scaling_factor_host(float amax, float old_scale, int fmt, int margin);
+
+/* out = saturating_rne_fp8(fp32(x) * *scale).  Replaces tex.cast_to_fp8
+ * (src/nanotron/fp8/tensor.py:65).  x is [rows, cols]; out_t, when not NULL, also receives the
+ * transposed bytes [cols, rows] (what tex.fp8_transpose, src/nanotron/fp8/kernel.py:43-44, would
+ * produce from `out`), written in the same pass. */
+int ntfp8_cast_to_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* scale,
+                      int fmt, void* out, void* out_t, void* stream);
+
+/* FP8Tensor.__new__ in one call (src/nanotron/fp8/tensor.py:25-28): current scaling.
+ * amax pass, scale from amax starting at 1.0, cast pass.  If amax_history is not NULL the
+ * delayed-scaling state is updated as well (history rolled, *scale_state = next scale), which
+ * is what the first use of a delayed-scaling role does. */
+int ntfp8_quantize_current(const void* x, int x_dtype, int64_t rows, int64_t cols, int fmt, int margin,
+                           float* amax_out, float* scale_used_out, void* out, void* out_t,
+                           float* amax_history, int history_len, float* scale_state,
+                           void* workspace, void* stream);
+
+/* One delayed-scaling step in a single pass over x (no counterpart in the reference, which
+ * has no amax history; semantics fixed by the benchmark configs: history 16, margin 0):
+ *   a = amax(x); q = cast(x, *scale_state); roll amax_history, hist[0] = a;
+ *   *scale_used_out = old *scale_state; *scale_state = update_scaling_factor(max(hist), old). */
+int ntfp8_quantize_delayed(const void* x, int x_dtype, int64_t rows, int64_t cols, int fmt, int margin,
+                           float* scale_state, float* amax_history, int history_len,
+                           float* amax_out, float* scale_used_out, void* out, void* out_t,
+                           void* workspace, void* stream);
+
+/* out = out_dtype(fp32(fp8) * (1 / *scale)).  Replaces tex.cast_from_fp8
+ * (src/nanotron/fp8/tensor.py:74) with meta.inverse_scale (src/nanotron/fp8/meta.py:36-37). */
+int ntfp8_cast_from_fp8(const void* in, int fmt, const float* scale, int64_t n, void* out, int out_dtype,
+                        void* stream);
+
+/* Byte transpose [rows, cols] -> [cols, rows].  Replaces tex.fp8_transpose
+ * (src/nanotron/fp8/kernel.py:43-44). */
+int ntfp8_transpose(const void* in, int64_t rows, int64_t cols, void* out, void* stream);
+
+/* D[M,N] (+)= (A[M,K] . B[N,K]^T) * (1 / *scale_a) * (1 / *scale_b), fp32 accumulation.
+ * Replaces tex.te_gemm in the only form the reference issues it (transa=True, transb=False:
+ * both operands contiguous along the reduction dimension; src/nanotron/fp8/kernel.py:46-68).
+ * d_dtype: NTFP8_F32 (reference default, kernel.py:24,28), NTFP8_BF16 or NTFP8_F16.
+ * accumulate != 0 adds into D (fp32 only) before the single rounding: the fp32 master-gradient
+ * accumulation of src/nanotron/optim/gradient_accumulator.py:222 folded into the epilogue. */
+int ntfp8_gemm(const void* A, int fmt_a, const float* scale_a,
+               const void* B, int fmt_b, const float* scale_b,
+               void* D, int d_dtype, int64_t M, int64_t N, int64_t K, int accumulate, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NTFP8_H */

@@ -1,0 +1,92 @@
+"""ctypes binding of libntfp8.so, the C-ABI library declared in include/ntfp8.h.
+
+There is no fallback: if the library is missing the import fails, and every wrapper turns a
+non-zero return code into a RuntimeError.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Dict, Optional, Tuple
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libntfp8.so")
+
+E4M3, E5M2 = 0, 1
+F32, F16, BF16 = 0, 1, 2
+WORKSPACE_BYTES = 64
+
+TORCH_TO_NT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        f"{LIB_PATH} is missing: build the HIP library first (python -m nanotron_amd.build). "
+        "nanotron_amd has no CPU or PyTorch fallback for its kernels."
+    )
+
+_lib = ctypes.CDLL(LIB_PATH)
+
+_c = ctypes
+_vp, _i, _i64, _f = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_float
+
+SIGNATURES = {
+    "ntfp8_version": (_i, []),
+    "ntfp8_strerror": (_c.c_char_p, [_i]),
+    "ntfp8_amax_scale": (_i, [_vp, _i, _i64, _i, _i, _vp, _vp, _vp, _vp, _vp]),
+    "ntfp8_update_scaling_factor": (_i, [_vp, _vp, _i, _i, _vp, _i64, _vp]),
+    "ntfp8_update_scaling_factor_host": (_f, [_f, _f, _i, _i]),
+    "ntfp8_cast_to_fp8": (_i, [_vp, _i, _i64, _i64, _vp, _i, _vp, _vp, _vp]),
+    "ntfp8_quantize_current": (_i, [_vp, _i, _i64, _i64, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp]),
+    "ntfp8_quantize_delayed": (_i, [_vp, _i, _i64, _i64, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "ntfp8_cast_from_fp8": (_i, [_vp, _i, _vp, _i64, _vp, _i, _vp]),
+    "ntfp8_transpose": (_i, [_vp, _i64, _i64, _vp, _vp]),
+    "ntfp8_gemm": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i64, _i64, _i64, _i, _vp]),
+}
+
+for _name, (_res, _args) in SIGNATURES.items():
+    _fn = getattr(_lib, _name)  # AttributeError here = library / header mismatch
+    _fn.restype = _res
+    _fn.argtypes = _args
+
+lib = _lib
+
+
+def strerror(code: int) -> str:
+    return _lib.ntfp8_strerror(code).decode()
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        raise RuntimeError(f"{what} failed: {strerror(code)} (code {code})")
+
+
+def version() -> int:
+    return _lib.ntfp8_version()
+
+
+def stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def workspace(device: torch.device) -> torch.Tensor:
+    """Zero-initialised reduction workspace, one per (device, stream): kernels leave it zero."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    key = (idx, stream_ptr(device))
+    ws = _workspaces.get(key)
+    if ws is None:
+        ws = torch.zeros(WORKSPACE_BYTES // 4, dtype=torch.int32, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def update_scaling_factor_host(amax: float, old: float, fmt: int, margin: int) -> float:
+    return float(_lib.ntfp8_update_scaling_factor_host(amax, old, fmt, margin))

@@ -1,0 +1,200 @@
+// extern "C" entry points declared in include/ntfp8.h: argument validation on the host, then one or
+// two kernel launches on the caller's stream.  Nothing here allocates, frees or synchronises.
+#include "common.h"
+
+namespace ntfp8 {
+
+int run_quant(int mode, const void* x, int x_dtype, int64_t rows, int64_t cols, int fmt, uint8_t* out, uint8_t* out_t,
+              const float* scale_ptr, Workspace* ws, const ScalarIO& io, hipStream_t st);
+int run_dequant(const void* in, int fmt, const float* scale, int64_t n, void* out, int out_dtype, hipStream_t st);
+int run_transpose(const void* in, int64_t rows, int64_t cols, void* out, hipStream_t st);
+int run_update_scale(const float* amax, const float* old_scale, int fmt, int margin, float* out, int64_t n,
+                     hipStream_t st);
+int run_gemm(const void* A, int fmt_a, const float* sa, const void* B, int fmt_b, const float* sb, void* D, int d_dtype,
+             int M, int N, int K, int accumulate, hipStream_t st);
+
+namespace {
+
+constexpr int kMaxHistory = 65536;
+constexpr int kMaxMargin = 126;
+
+bool fmt_ok(int f) { return f == NTFP8_E4M3 || f == NTFP8_E5M2; }
+bool dtype_ok(int d) { return d == NTFP8_F32 || d == NTFP8_F16 || d == NTFP8_BF16; }
+size_t dtype_size(int d) { return d == NTFP8_F32 ? 4 : 2; }
+bool is_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+// rows * cols as a positive int64, or false
+bool numel(int64_t rows, int64_t cols, int64_t* n) {
+    if (rows <= 0 || cols <= 0) return false;
+    long long r;
+    if (__builtin_smulll_overflow((long long)rows, (long long)cols, &r)) return false;
+    if (r > (1LL << 46)) return false;
+    *n = r;
+    return true;
+}
+
+bool overlap(const void* a, size_t an, const void* b, size_t bn) {
+    const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+    return a0 < b0 + bn && b0 < a0 + an;
+}
+
+int check_quant_common(const void* x, int x_dtype, int64_t rows, int64_t cols, int fmt, int margin, int64_t* n) {
+    if (!x) return NTFP8_ERR_NULL;
+    if (!fmt_ok(fmt) || !dtype_ok(x_dtype)) return NTFP8_ERR_ENUM;
+    if (!numel(rows, cols, n)) return NTFP8_ERR_SIZE;
+    if (margin < -kMaxMargin || margin > kMaxMargin) return NTFP8_ERR_SIZE;
+    if (!is_aligned(x, dtype_size(x_dtype))) return NTFP8_ERR_ALIGN;
+    return NTFP8_OK;
+}
+
+int check_outputs(const void* x, int x_dtype, int64_t n, const void* out, const void* out_t) {
+    const size_t xb = (size_t)n * dtype_size(x_dtype);
+    if (out && overlap(x, xb, out, (size_t)n)) return NTFP8_ERR_ALIAS;
+    if (out_t && overlap(x, xb, out_t, (size_t)n)) return NTFP8_ERR_ALIAS;
+    if (out && out_t && overlap(out, (size_t)n, out_t, (size_t)n)) return NTFP8_ERR_ALIAS;
+    return NTFP8_OK;
+}
+
+}  // namespace
+}  // namespace ntfp8
+
+using namespace ntfp8;
+
+extern "C" {
+
+int ntfp8_version(void) { return NTFP8_VERSION; }
+
+const char* ntfp8_strerror(int code) {
+    switch (code) {
+        case NTFP8_OK: return "ok";
+        case NTFP8_ERR_NULL: return "a required pointer is NULL";
+        case NTFP8_ERR_ENUM: return "unknown format or dtype";
+        case NTFP8_ERR_SIZE: return "size, history length or margin out of range";
+        case NTFP8_ERR_ALIGN: return "pointer is not aligned to its element type";
+        case NTFP8_ERR_UNSUPPORTED: return "request not supported";
+        case NTFP8_ERR_LAUNCH: return "HIP reported an error at kernel launch";
+        case NTFP8_ERR_ALIAS: return "an output overlaps an input or another output";
+        default: return "unknown error code";
+    }
+}
+
+int ntfp8_amax_scale(const void* x, int x_dtype, int64_t n, int fmt, int margin, const float* old_scale,
+                     float* amax_out, float* scale_out, void* workspace, void* stream) {
+    int64_t nn;
+    if (!amax_out || !scale_out || !workspace) return NTFP8_ERR_NULL;
+    int rc = check_quant_common(x, x_dtype, n, 1, fmt, margin, &nn);
+    if (rc) return rc;
+    if (!is_aligned(amax_out, 4) || !is_aligned(scale_out, 4) || !is_aligned(workspace, 4) ||
+        (old_scale && !is_aligned(old_scale, 4)))
+        return NTFP8_ERR_ALIGN;
+    ScalarIO io = {old_scale, amax_out, scale_out, nullptr, nullptr, 0, fmt, margin};
+    return run_quant(kModeAmaxOnly, x, x_dtype, nn, 1, fmt, nullptr, nullptr, nullptr, static_cast<Workspace*>(workspace),
+                     io, static_cast<hipStream_t>(stream));
+}
+
+int ntfp8_update_scaling_factor(const float* amax, const float* old_scale, int fmt, int margin, float* out, int64_t n,
+                                void* stream) {
+    if (!amax || !old_scale || !out) return NTFP8_ERR_NULL;
+    if (!fmt_ok(fmt)) return NTFP8_ERR_ENUM;
+    if (n <= 0 || n > (1LL << 40) || margin < -kMaxMargin || margin > kMaxMargin) return NTFP8_ERR_SIZE;
+    if (!is_aligned(amax, 4) || !is_aligned(old_scale, 4) || !is_aligned(out, 4)) return NTFP8_ERR_ALIGN;
+    return run_update_scale(amax, old_scale, fmt, margin, out, n, static_cast<hipStream_t>(stream));
+}
+
+float ntfp8_update_scaling_factor_host(float amax, float old_scale, int fmt, int margin) {
+    if (!fmt_ok(fmt) || margin < -kMaxMargin || margin > kMaxMargin) return bits_f32(kNanBits);
+    return update_scale(amax, old_scale, fmt, margin);
+}
+
+int ntfp8_cast_to_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* scale, int fmt, void* out,
+                      void* out_t, void* stream) {
+    int64_t n;
+    if (!scale || (!out && !out_t)) return NTFP8_ERR_NULL;
+    int rc = check_quant_common(x, x_dtype, rows, cols, fmt, 0, &n);
+    if (rc) return rc;
+    if (!is_aligned(scale, 4)) return NTFP8_ERR_ALIGN;
+    rc = check_outputs(x, x_dtype, n, out, out_t);
+    if (rc) return rc;
+    ScalarIO io = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, fmt, 0};
+    return run_quant(kModeCastOnly, x, x_dtype, rows, cols, fmt, static_cast<uint8_t*>(out), static_cast<uint8_t*>(out_t),
+                     scale, nullptr, io, static_cast<hipStream_t>(stream));
+}
+
+int ntfp8_quantize_current(const void* x, int x_dtype, int64_t rows, int64_t cols, int fmt, int margin, float* amax_out,
+                           float* scale_used_out, void* out, void* out_t, float* amax_history, int history_len,
+                           float* scale_state, void* workspace, void* stream) {
+    int64_t n;
+    if (!amax_out || !scale_used_out || !workspace || (!out && !out_t)) return NTFP8_ERR_NULL;
+    int rc = check_quant_common(x, x_dtype, rows, cols, fmt, margin, &n);
+    if (rc) return rc;
+    if (amax_history) {
+        if (!scale_state) return NTFP8_ERR_NULL;
+        if (history_len < 1 || history_len > kMaxHistory) return NTFP8_ERR_SIZE;
+        if (!is_aligned(amax_history, 4) || !is_aligned(scale_state, 4)) return NTFP8_ERR_ALIGN;
+    }
+    if (!is_aligned(amax_out, 4) || !is_aligned(scale_used_out, 4) || !is_aligned(workspace, 4)) return NTFP8_ERR_ALIGN;
+    rc = check_outputs(x, x_dtype, n, out, out_t);
+    if (rc) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    ScalarIO io = {nullptr, amax_out, scale_used_out, amax_history ? scale_state : nullptr, amax_history,
+                   amax_history ? history_len : 0, fmt, margin};
+    rc = run_quant(kModeAmaxOnly, x, x_dtype, n, 1, fmt, nullptr, nullptr, nullptr, static_cast<Workspace*>(workspace), io,
+                   st);
+    if (rc) return rc;
+    ScalarIO none = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, fmt, 0};
+    return run_quant(kModeCastOnly, x, x_dtype, rows, cols, fmt, static_cast<uint8_t*>(out), static_cast<uint8_t*>(out_t),
+                     scale_used_out, nullptr, none, st);
+}
+
+int ntfp8_quantize_delayed(const void* x, int x_dtype, int64_t rows, int64_t cols, int fmt, int margin,
+                           float* scale_state, float* amax_history, int history_len, float* amax_out,
+                           float* scale_used_out, void* out, void* out_t, void* workspace, void* stream) {
+    int64_t n;
+    if (!scale_state || !amax_history || !amax_out || !workspace || (!out && !out_t)) return NTFP8_ERR_NULL;
+    int rc = check_quant_common(x, x_dtype, rows, cols, fmt, margin, &n);
+    if (rc) return rc;
+    if (history_len < 1 || history_len > kMaxHistory) return NTFP8_ERR_SIZE;
+    if (!is_aligned(scale_state, 4) || !is_aligned(amax_history, 4) || !is_aligned(amax_out, 4) ||
+        !is_aligned(workspace, 4) || (scale_used_out && !is_aligned(scale_used_out, 4)))
+        return NTFP8_ERR_ALIGN;
+    rc = check_outputs(x, x_dtype, n, out, out_t);
+    if (rc) return rc;
+    ScalarIO io = {nullptr, amax_out, scale_used_out, scale_state, amax_history, history_len, fmt, margin};
+    return run_quant(kModeDelayed, x, x_dtype, rows, cols, fmt, static_cast<uint8_t*>(out), static_cast<uint8_t*>(out_t),
+                     scale_state, static_cast<Workspace*>(workspace), io, static_cast<hipStream_t>(stream));
+}
+
+int ntfp8_cast_from_fp8(const void* in, int fmt, const float* scale, int64_t n, void* out, int out_dtype, void* stream) {
+    if (!in || !scale || !out) return NTFP8_ERR_NULL;
+    if (!fmt_ok(fmt) || !dtype_ok(out_dtype)) return NTFP8_ERR_ENUM;
+    if (n <= 0 || n > (1LL << 46)) return NTFP8_ERR_SIZE;
+    if (!is_aligned(scale, 4) || !is_aligned(out, dtype_size(out_dtype))) return NTFP8_ERR_ALIGN;
+    if (overlap(in, (size_t)n, out, (size_t)n * dtype_size(out_dtype))) return NTFP8_ERR_ALIAS;
+    return run_dequant(in, fmt, scale, n, out, out_dtype, static_cast<hipStream_t>(stream));
+}
+
+int ntfp8_transpose(const void* in, int64_t rows, int64_t cols, void* out, void* stream) {
+    int64_t n;
+    if (!in || !out) return NTFP8_ERR_NULL;
+    if (!numel(rows, cols, &n)) return NTFP8_ERR_SIZE;
+    if (overlap(in, (size_t)n, out, (size_t)n)) return NTFP8_ERR_ALIAS;
+    return run_transpose(in, rows, cols, out, static_cast<hipStream_t>(stream));
+}
+
+int ntfp8_gemm(const void* A, int fmt_a, const float* scale_a, const void* B, int fmt_b, const float* scale_b, void* D,
+               int d_dtype, int64_t M, int64_t N, int64_t K, int accumulate, void* stream) {
+    if (!A || !B || !D || !scale_a || !scale_b) return NTFP8_ERR_NULL;
+    if (!fmt_ok(fmt_a) || !fmt_ok(fmt_b) || !dtype_ok(d_dtype)) return NTFP8_ERR_ENUM;
+    if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffff00LL || N > 0x7fffff00LL || K > 0x7fffff00LL) return NTFP8_ERR_SIZE;
+    int64_t mn, mk, nk;
+    if (!numel(M, N, &mn) || !numel(M, K, &mk) || !numel(N, K, &nk)) return NTFP8_ERR_SIZE;
+    if (((M + 127) / 128) * ((N + 127) / 128) > 0x7fffffffLL) return NTFP8_ERR_SIZE;
+    if (accumulate && d_dtype != NTFP8_F32) return NTFP8_ERR_UNSUPPORTED;
+    if (!is_aligned(scale_a, 4) || !is_aligned(scale_b, 4) || !is_aligned(D, dtype_size(d_dtype))) return NTFP8_ERR_ALIGN;
+    const size_t db = (size_t)mn * dtype_size(d_dtype);
+    if (overlap(A, (size_t)mk, D, db) || overlap(B, (size_t)nk, D, db)) return NTFP8_ERR_ALIAS;
+    return run_gemm(A, fmt_a, scale_a, B, fmt_b, scale_b, D, d_dtype, (int)M, (int)N, (int)K, accumulate,
+                    static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,501 @@
+// amax reduction, delayed-scaling history roll + scale update, saturating casts to OCP FP8,
+// dequantisation and byte transpose for gfx950.  All kernels are HBM-bandwidth bound: one pass
+// over the input with 128-bit loads and stores, a wavefront reduction for the amax, one atomic per
+// block and a last-block epilogue that finishes the scalar bookkeeping in the same launch.
+#include "common.h"
+
+namespace ntfp8 {
+
+constexpr int kThreads = 256;
+constexpr int kVec = 16;  // elements per thread per step: 16 fp8 bytes = one 128-bit store
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+
+
+// ---------------------------------------------------------------------------------------------
+// 16-element loads.  `m16` receives max|x| of the 16 elements as a comparable unsigned pattern in
+// the *source* format (fp32 bits for float, 16-bit patterns for half / bf16).
+template <typename T>
+struct Src;
+
+template <>
+struct Src<float> {
+    static constexpr int kDtype = NTFP8_F32;
+    __device__ static __forceinline__ void load16(const float* p, float (&v)[16], uint32_t& m16) {
+        const f4* q = reinterpret_cast<const f4*>(p);
+        uint32_t m = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const f4 t = __builtin_nontemporal_load(q + i);
+            v[4 * i + 0] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t a = __float_as_uint(v[i]) & 0x7fffffffu;
+            m = a > m ? a : m;
+        }
+        m16 = m;
+    }
+    __device__ static __forceinline__ float load1(const float* p, uint32_t& m) {
+        const float x = *p;
+        m = __float_as_uint(x) & 0x7fffffffu;
+        return x;
+    }
+    __device__ static __forceinline__ bool has_nan(uint32_t m) { return m > kInfBits; }
+    __device__ static __forceinline__ uint32_t to_f32_bits(uint32_t m) { return m; }
+};
+
+template <bool kBf16>
+struct Src16 {
+    __device__ static __forceinline__ float cvt(uint32_t h) {
+        if constexpr (kBf16) return bf16_bits_to_float(h);
+        else return half_bits_to_float(h);
+    }
+    __device__ static __forceinline__ void load16(const uint16_t* p, float (&v)[16], uint32_t& m16) {
+        const u4* q = reinterpret_cast<const u4*>(p);
+        const u4 a = __builtin_nontemporal_load(q);
+        const u4 b = __builtin_nontemporal_load(q + 1);
+        const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+        us2 m = {0, 0};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if constexpr (kBf16) {
+                v[2 * i] = __uint_as_float(w[i] << 16);
+                v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+            } else {
+                v[2 * i] = half_bits_to_float(w[i] & 0xffffu);
+                v[2 * i + 1] = half_bits_to_float(w[i] >> 16);
+            }
+            const uint32_t ab = w[i] & 0x7fff7fffu;
+            us2 t;
+            __builtin_memcpy(&t, &ab, 4);
+            m = __builtin_elementwise_max(m, t);
+        }
+        m16 = m.x > m.y ? m.x : m.y;
+    }
+    __device__ static __forceinline__ float load1(const uint16_t* p, uint32_t& m) {
+        const uint32_t h = *p;
+        m = h & 0x7fffu;
+        return cvt(h);
+    }
+    __device__ static __forceinline__ bool has_nan(uint32_t m) { return m > (kBf16 ? 0x7f80u : 0x7c00u); }
+    __device__ static __forceinline__ uint32_t to_f32_bits(uint32_t m) { return __float_as_uint(cvt(m)); }
+};
+
+struct bf16_tag {};
+struct f16_tag {};
+template <>
+struct Src<bf16_tag> : Src16<true> {
+    static constexpr int kDtype = NTFP8_BF16;
+    typedef uint16_t elem;
+};
+template <>
+struct Src<f16_tag> : Src16<false> {
+    static constexpr int kDtype = NTFP8_F16;
+    typedef uint16_t elem;
+};
+template <typename T>
+struct ElemOf {
+    typedef uint16_t type;
+};
+template <>
+struct ElemOf<float> {
+    typedef float type;
+};
+
+// 16 scaled values -> 16 fp8 bytes.  `slow` = this group may contain a NaN (NaN input or a
+// degenerate scale): patch the NaN bytes to sign|0x7F.
+template <int F>
+__device__ __forceinline__ u4 encode16(const float (&v)[16], float scale, bool slow) {
+    float y[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) y[i] = v[i] * scale;
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        w[i] = cvt4<F>(sat<F>(y[4 * i]), sat<F>(y[4 * i + 1]), sat<F>(y[4 * i + 2]), sat<F>(y[4 * i + 3]));
+    if (slow) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) w[i >> 2] = patch_nan(w[i >> 2], i & 3, y[i]);
+    }
+    return (u4){w[0], w[1], w[2], w[3]};
+}
+
+template <int F>
+__device__ __forceinline__ uint8_t encode1(float x, float scale) {
+    const float y = x * scale;
+    uint32_t w = cvt4<F>(sat<F>(y), 0.0f, 0.0f, 0.0f);
+    w = patch_nan(w, 0, y);
+    return (uint8_t)(w & 0xffu);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Block reduction of the partial max, publication, and the last-block epilogue.
+__device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, const ScalarIO& io, int mode) {
+    __shared__ uint32_t s_part[kThreads / 64];
+    __shared__ bool s_last;
+    const uint32_t wm = wave_max_u32(m_f32bits);
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = wm;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t bm = 0;
+#pragma unroll
+        for (int i = 0; i < kThreads / 64; ++i) bm = s_part[i] > bm ? s_part[i] : bm;
+        if (bm) __hip_atomic_fetch_max(&ws->amax_bits, bm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __threadfence();
+        const uint32_t t = __hip_atomic_fetch_add(&ws->ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (t == gridDim.x - 1);
+    }
+    __syncthreads();
+    if (!s_last || threadIdx.x != 0) return;
+    __threadfence();
+    uint32_t bits = __hip_atomic_load(&ws->amax_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (bits > kInfBits) bits = kNanBits;
+    const float a = __uint_as_float(bits);
+    *io.amax_out = a;
+    float used;
+    if (mode == kModeAmaxOnly) {
+        const float old = io.old_scale ? *io.old_scale : 1.0f;
+        used = update_scale(a, old, io.fmt, io.margin);
+    } else {
+        used = *io.scale_state;
+    }
+    if (io.scale_out) *io.scale_out = used;
+    if (io.hist) {
+        uint32_t hm = bits;
+        for (int i = io.hist_len - 1; i > 0; --i) {
+            const float h = io.hist[i - 1];
+            io.hist[i] = h;
+            uint32_t hb = __float_as_uint(h) & 0x7fffffffu;
+            hm = hb > hm ? hb : hm;
+        }
+        io.hist[0] = a;
+        if (hm > kInfBits) hm = kNanBits;
+        *io.scale_state = update_scale(__uint_as_float(hm), used, io.fmt, io.margin);
+    }
+    __hip_atomic_store(&ws->amax_bits, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&ws->ticket, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ bool degenerate_scale(float s) {
+    const uint32_t b = __float_as_uint(s) & 0x7fffffffu;
+    return b == 0u || b >= kInfBits;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Flat (no transpose) kernel: amax only, cast only, or both (delayed scaling).
+template <typename S, int F, int MODE>
+__global__ __launch_bounds__(kThreads) void quant_flat_kernel(const typename ElemOf<S>::type* __restrict__ x,
+                                                              int64_t n_vec, int64_t n, uint8_t* __restrict__ out,
+                                                              const float* __restrict__ scale_ptr, Workspace* ws,
+                                                              ScalarIO io) {
+    typedef Src<S> L;
+    constexpr bool kCast = MODE != kModeAmaxOnly;
+    constexpr bool kAmax = MODE != kModeCastOnly;
+    float scale = 1.0f;
+    bool degen = false;
+    if constexpr (kCast) {
+        scale = *scale_ptr;
+        degen = degenerate_scale(scale);
+    }
+    uint32_t m_run = 0;  // in source-format bits
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    // two groups per trip: four (bf16) or eight (fp32) 128-bit loads in flight per lane
+    for (; i + stride < n_vec; i += 2 * stride) {
+        float v0[16], v1[16];
+        uint32_t m0, m1;
+        L::load16(x + i * kVec, v0, m0);
+        L::load16(x + (i + stride) * kVec, v1, m1);
+        if constexpr (kAmax) {
+            m_run = m0 > m_run ? m0 : m_run;
+            m_run = m1 > m_run ? m1 : m_run;
+        }
+        if constexpr (kCast) {
+            const u4 q0 = encode16<F>(v0, scale, degen || L::has_nan(m0));
+            const u4 q1 = encode16<F>(v1, scale, degen || L::has_nan(m1));
+            __builtin_nontemporal_store(q0, reinterpret_cast<u4*>(out + i * kVec));
+            __builtin_nontemporal_store(q1, reinterpret_cast<u4*>(out + (i + stride) * kVec));
+        }
+    }
+    if (i < n_vec) {
+        float v0[16];
+        uint32_t m0;
+        L::load16(x + i * kVec, v0, m0);
+        if constexpr (kAmax) m_run = m0 > m_run ? m0 : m_run;
+        if constexpr (kCast) {
+            const u4 q0 = encode16<F>(v0, scale, degen || L::has_nan(m0));
+            __builtin_nontemporal_store(q0, reinterpret_cast<u4*>(out + i * kVec));
+        }
+    }
+    // elements the vector body does not cover (tail, or everything when a pointer is misaligned)
+    for (int64_t j = n_vec * kVec + (int64_t)blockIdx.x * kThreads + threadIdx.x; j < n; j += stride) {
+        uint32_t m;
+        const float xv = L::load1(x + j, m);
+        if constexpr (kAmax) m_run = m > m_run ? m : m_run;
+        if constexpr (kCast) out[j] = encode1<F>(xv, scale);
+    }
+    if constexpr (kAmax) publish_and_finalize(L::to_f32_bits(m_run), ws, io, MODE);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Cast (+ optional amax) that also writes the transposed bytes.  One 128x128 tile per block, staged
+// through 16 KB of LDS.  LDS holds the tile transposed, [col][row], the 16-byte row chunks of each
+// column XOR-swizzled with the column's 16-wide chunk index so that both the byte stores of phase 1
+// and the 128-bit loads of phase 2 are bank-conflict free.
+constexpr int kTile = 128;
+
+template <typename S, int F, bool kAmax>
+__global__ __launch_bounds__(kThreads) void quant_transpose_kernel(const typename ElemOf<S>::type* __restrict__ x,
+                                                                   int64_t rows, int64_t cols,
+                                                                   uint8_t* __restrict__ out,
+                                                                   uint8_t* __restrict__ out_t,
+                                                                   const float* __restrict__ scale_ptr,
+                                                                   Workspace* ws, ScalarIO io) {
+    typedef Src<S> L;
+    __shared__ __attribute__((aligned(16))) uint8_t tile[kTile * kTile];
+    const float scale = *scale_ptr;
+    const bool degen = degenerate_scale(scale);
+    const int64_t tiles_c = cols / kTile;
+    const int64_t tr = blockIdx.x / tiles_c, tc = blockIdx.x % tiles_c;
+    const int64_t row0 = tr * kTile, col0 = tc * kTile;
+    const int t = threadIdx.x;
+    const int cchunk = t & 7;   // 16-column chunk inside the tile
+    const int rsub = t >> 3;    // 0..31
+    uint32_t m_run = 0;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int r = rsub + 32 * it;
+        const int64_t g = (row0 + r) * cols + col0 + cchunk * 16;
+        float v[16];
+        uint32_t m16;
+        L::load16(x + g, v, m16);
+        if constexpr (kAmax) m_run = m16 > m_run ? m16 : m_run;
+        const u4 q = encode16<F>(v, scale, degen || L::has_nan(m16));
+        if (out) __builtin_nontemporal_store(q, reinterpret_cast<u4*>(out + g));
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+        const int rsw = r ^ (cchunk << 4);  // swizzled row position inside a column
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+            tile[(cchunk * 16 + j) * kTile + rsw] = (uint8_t)(w[j >> 2] >> (8 * (j & 3)));
+    }
+    __syncthreads();
+    const int rchunk = t & 7;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int c = rsub + 32 * it;
+        const int pos = (rchunk ^ (c >> 4)) << 4;
+        const u4 q = *reinterpret_cast<const u4*>(&tile[c * kTile + pos]);
+        __builtin_nontemporal_store(q, reinterpret_cast<u4*>(out_t + (col0 + c) * rows + row0 + rchunk * 16));
+    }
+    if constexpr (kAmax) publish_and_finalize(L::to_f32_bits(m_run), ws, io, kModeDelayed);
+}
+
+// Any shape: one element per thread step, transposed store.  Used when the tile kernel's
+// 128-multiples / alignment requirements are not met.
+template <typename S, int F, bool kAmax>
+__global__ __launch_bounds__(kThreads) void quant_transpose_scalar_kernel(
+    const typename ElemOf<S>::type* __restrict__ x, int64_t rows, int64_t cols, uint8_t* __restrict__ out,
+    uint8_t* __restrict__ out_t, const float* __restrict__ scale_ptr, Workspace* ws, ScalarIO io) {
+    typedef Src<S> L;
+    const float scale = *scale_ptr;
+    const int64_t n = rows * cols;
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    uint32_t m_run = 0;
+    for (int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x; j < n; j += stride) {
+        uint32_t m;
+        const float xv = L::load1(x + j, m);
+        if constexpr (kAmax) m_run = m > m_run ? m : m_run;
+        const uint8_t b = encode1<F>(xv, scale);
+        if (out) out[j] = b;
+        const int64_t r = j / cols, c = j % cols;
+        out_t[c * rows + r] = b;
+    }
+    if constexpr (kAmax) publish_and_finalize(L::to_f32_bits(m_run), ws, io, kModeDelayed);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Dequantise: out = out_dtype(decode(byte) * (1 / scale)).
+template <int F>
+__device__ __forceinline__ float decode1(uint32_t b) {
+    if constexpr (F == kE4M3) return __builtin_amdgcn_cvt_f32_fp8((int)b, 0);
+    else return __builtin_amdgcn_cvt_f32_bf8((int)b, 0);
+}
+
+template <int F, int OUT>
+__global__ __launch_bounds__(kThreads) void dequant_kernel(const uint8_t* __restrict__ in, int64_t n,
+                                                           const float* __restrict__ scale_ptr, void* __restrict__ out) {
+    const float inv = 1.0f / *scale_ptr;
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    for (int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x; j < n; j += stride) {
+        const float v = decode1<F>(in[j]) * inv;
+        if constexpr (OUT == NTFP8_F32) ((float*)out)[j] = v;
+        else if constexpr (OUT == NTFP8_F16) ((__half*)out)[j] = __float2half_rn(v);
+        else {
+            // bf16 round-to-nearest-even with NaN kept quiet
+            uint32_t u = __float_as_uint(v);
+            uint16_t r;
+            if ((u & 0x7fffffffu) > kInfBits) r = (uint16_t)((u >> 16) | 0x40u);
+            else r = (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+            ((uint16_t*)out)[j] = r;
+        }
+    }
+}
+
+// Byte transpose through a 64x64 LDS tile (pitch 65 breaks the bank pattern); any shape.
+__global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __restrict__ in, int64_t rows, int64_t cols,
+                                                             uint8_t* __restrict__ out) {
+    __shared__ uint8_t tile[64][65];
+    const int64_t tiles_c = (cols + 63) / 64;
+    const int64_t r0 = (blockIdx.x / tiles_c) * 64, c0 = (blockIdx.x % tiles_c) * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int r = ty; r < 64; r += 4)
+        if (r0 + r < rows && c0 + tx < cols) tile[r][tx] = in[(r0 + r) * cols + c0 + tx];
+    __syncthreads();
+    for (int c = ty; c < 64; c += 4)
+        if (c0 + c < cols && r0 + tx < rows) out[(c0 + c) * rows + r0 + tx] = tile[tx][c];
+}
+
+__global__ void update_scale_kernel(const float* amax, const float* old_scale, int fmt, int margin, float* out,
+                                    int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = update_scale(amax[i], old_scale[i], fmt, margin);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host-side launchers.
+static int grid_for(int64_t work_items, int per_cu_blocks = 8) {
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
+    }
+    int64_t want = (work_items + kThreads - 1) / kThreads;
+    int64_t cap = (int64_t)cus * per_cu_blocks;
+    if (want < 1) want = 1;
+    return (int)(want < cap ? want : cap);
+}
+
+static int check_launch() { return hipGetLastError() == hipSuccess ? NTFP8_OK : NTFP8_ERR_LAUNCH; }
+
+template <typename S, int F>
+static int launch_flat(int mode, const void* x, int64_t n, bool vec_ok, uint8_t* out, const float* scale_ptr,
+                       Workspace* ws, const ScalarIO& io, hipStream_t st) {
+    typedef typename ElemOf<S>::type E;
+    const int64_t n_vec = vec_ok ? n / kVec : 0;
+    // two 16-element groups per lane per trip
+    const int grid = grid_for(n_vec > 0 ? (n_vec + 1) / 2 : n);
+    const E* xp = static_cast<const E*>(x);
+    if (mode == kModeAmaxOnly)
+        hipLaunchKernelGGL((quant_flat_kernel<S, F, kModeAmaxOnly>), dim3(grid), dim3(kThreads), 0, st, xp, n_vec, n, out,
+                           scale_ptr, ws, io);
+    else if (mode == kModeCastOnly)
+        hipLaunchKernelGGL((quant_flat_kernel<S, F, kModeCastOnly>), dim3(grid), dim3(kThreads), 0, st, xp, n_vec, n, out,
+                           scale_ptr, ws, io);
+    else
+        hipLaunchKernelGGL((quant_flat_kernel<S, F, kModeDelayed>), dim3(grid), dim3(kThreads), 0, st, xp, n_vec, n, out,
+                           scale_ptr, ws, io);
+    return check_launch();
+}
+
+template <typename S, int F>
+static int launch_transpose(bool with_amax, const void* x, int64_t rows, int64_t cols, bool tile_ok, uint8_t* out,
+                            uint8_t* out_t, const float* scale_ptr, Workspace* ws, const ScalarIO& io, hipStream_t st) {
+    typedef typename ElemOf<S>::type E;
+    const E* xp = static_cast<const E*>(x);
+    if (tile_ok) {
+        const int64_t tiles = (rows / kTile) * (cols / kTile);
+        if (tiles > 0x7fffffff) return NTFP8_ERR_SIZE;
+        if (with_amax)
+            hipLaunchKernelGGL((quant_transpose_kernel<S, F, true>), dim3((int)tiles), dim3(kThreads), 0, st, xp, rows,
+                               cols, out, out_t, scale_ptr, ws, io);
+        else
+            hipLaunchKernelGGL((quant_transpose_kernel<S, F, false>), dim3((int)tiles), dim3(kThreads), 0, st, xp, rows,
+                               cols, out, out_t, scale_ptr, ws, io);
+    } else {
+        const int grid = grid_for(rows * cols);
+        if (with_amax)
+            hipLaunchKernelGGL((quant_transpose_scalar_kernel<S, F, true>), dim3(grid), dim3(kThreads), 0, st, xp, rows,
+                               cols, out, out_t, scale_ptr, ws, io);
+        else
+            hipLaunchKernelGGL((quant_transpose_scalar_kernel<S, F, false>), dim3(grid), dim3(kThreads), 0, st, xp, rows,
+                               cols, out, out_t, scale_ptr, ws, io);
+    }
+    return check_launch();
+}
+
+template <typename S>
+static int dispatch_fmt_flat(int fmt, int mode, const void* x, int64_t n, bool vec_ok, uint8_t* out,
+                             const float* scale_ptr, Workspace* ws, const ScalarIO& io, hipStream_t st) {
+    return fmt == kE4M3 ? launch_flat<S, kE4M3>(mode, x, n, vec_ok, out, scale_ptr, ws, io, st)
+                        : launch_flat<S, kE5M2>(mode, x, n, vec_ok, out, scale_ptr, ws, io, st);
+}
+
+template <typename S>
+static int dispatch_fmt_tr(int fmt, bool with_amax, const void* x, int64_t rows, int64_t cols, bool tile_ok,
+                           uint8_t* out, uint8_t* out_t, const float* scale_ptr, Workspace* ws, const ScalarIO& io,
+                           hipStream_t st) {
+    return fmt == kE4M3 ? launch_transpose<S, kE4M3>(with_amax, x, rows, cols, tile_ok, out, out_t, scale_ptr, ws, io, st)
+                        : launch_transpose<S, kE5M2>(with_amax, x, rows, cols, tile_ok, out, out_t, scale_ptr, ws, io, st);
+}
+
+static bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// mode: kModeAmaxOnly / kModeCastOnly / kModeDelayed.  out_t may be NULL.
+int run_quant(int mode, const void* x, int x_dtype, int64_t rows, int64_t cols, int fmt, uint8_t* out, uint8_t* out_t,
+              const float* scale_ptr, Workspace* ws, const ScalarIO& io, hipStream_t st) {
+    const int64_t n = rows * cols;
+    if (mode != kModeAmaxOnly && out_t != nullptr) {
+        const bool tile_ok = rows % kTile == 0 && cols % kTile == 0 && aligned(x, 16) && aligned(out_t, 16) &&
+                             (out == nullptr || aligned(out, 16));
+        const bool with_amax = mode == kModeDelayed;
+        switch (x_dtype) {
+            case NTFP8_F32: return dispatch_fmt_tr<float>(fmt, with_amax, x, rows, cols, tile_ok, out, out_t, scale_ptr, ws, io, st);
+            case NTFP8_F16: return dispatch_fmt_tr<f16_tag>(fmt, with_amax, x, rows, cols, tile_ok, out, out_t, scale_ptr, ws, io, st);
+            default: return dispatch_fmt_tr<bf16_tag>(fmt, with_amax, x, rows, cols, tile_ok, out, out_t, scale_ptr, ws, io, st);
+        }
+    }
+    const bool vec_ok = aligned(x, 16) && (mode == kModeAmaxOnly || aligned(out, 16));
+    switch (x_dtype) {
+        case NTFP8_F32: return dispatch_fmt_flat<float>(fmt, mode, x, n, vec_ok, out, scale_ptr, ws, io, st);
+        case NTFP8_F16: return dispatch_fmt_flat<f16_tag>(fmt, mode, x, n, vec_ok, out, scale_ptr, ws, io, st);
+        default: return dispatch_fmt_flat<bf16_tag>(fmt, mode, x, n, vec_ok, out, scale_ptr, ws, io, st);
+    }
+}
+
+int run_dequant(const void* in, int fmt, const float* scale, int64_t n, void* out, int out_dtype, hipStream_t st) {
+    const int grid = grid_for(n);
+    const uint8_t* p = static_cast<const uint8_t*>(in);
+#define NT_DQ(F, O) hipLaunchKernelGGL((dequant_kernel<F, O>), dim3(grid), dim3(kThreads), 0, st, p, n, scale, out)
+    if (fmt == kE4M3) {
+        if (out_dtype == NTFP8_F32) NT_DQ(kE4M3, NTFP8_F32);
+        else if (out_dtype == NTFP8_F16) NT_DQ(kE4M3, NTFP8_F16);
+        else NT_DQ(kE4M3, NTFP8_BF16);
+    } else {
+        if (out_dtype == NTFP8_F32) NT_DQ(kE5M2, NTFP8_F32);
+        else if (out_dtype == NTFP8_F16) NT_DQ(kE5M2, NTFP8_F16);
+        else NT_DQ(kE5M2, NTFP8_BF16);
+    }
+#undef NT_DQ
+    return check_launch();
+}
+
+int run_transpose(const void* in, int64_t rows, int64_t cols, void* out, hipStream_t st) {
+    const int64_t tiles = ((rows + 63) / 64) * ((cols + 63) / 64);
+    if (tiles > 0x7fffffff) return NTFP8_ERR_SIZE;
+    hipLaunchKernelGGL(transpose_kernel, dim3((int)tiles), dim3(kThreads), 0, st, static_cast<const uint8_t*>(in), rows,
+                       cols, static_cast<uint8_t*>(out));
+    return check_launch();
+}
+
+int run_update_scale(const float* amax, const float* old_scale, int fmt, int margin, float* out, int64_t n,
+                     hipStream_t st) {
+    const int64_t blocks = (n + 255) / 256;
+    if (blocks > 0x7fffffff) return NTFP8_ERR_SIZE;
+    hipLaunchKernelGGL(update_scale_kernel, dim3((int)blocks), dim3(256), 0, st, amax, old_scale, fmt, margin, out, n);
+    return check_launch();
+}
+
+}  // namespace ntfp8

@@ -1,0 +1,242 @@
+"""FP8Tensor and the quantise / dequantise entry points (reference: src/nanotron/fp8/tensor.py).
+
+The reference computes `amax` with two torch passes, the scale with ~8 scalar kernels and the cast
+with Transformer Engine.  Here one C-ABI call does all of it on the device; amax, scale and the
+delayed-scaling history never leave device memory.
+"""
+from __future__ import annotations
+
+from typing import Optional, Union
+
+import torch
+
+from nanotron_amd import _native as nt
+from nanotron_amd.fp8.constants import (
+    DEFAULT_AMAX_HISTORY_LEN,
+    DEFAULT_MARGIN,
+    FP8_DTYPES,
+    INITIAL_SCALING_FACTOR,
+)
+from nanotron_amd.fp8.dtypes import DType, DTypes
+
+_FMT = {DTypes.FP8E4M3: nt.E4M3, DTypes.FP8E5M2: nt.E5M2}
+
+
+def _int_margin(margin) -> int:
+    m = float(margin)
+    if not m.is_integer():
+        raise ValueError(f"margin must be an integer number of binades, got {margin}")
+    return int(m)
+
+
+class DelayedScaling:
+    """Per tensor-role delayed-scaling state kept on the device: `scale` (the scale the NEXT
+    quantisation will use) and `amax_history` (newest first).  Not in the reference, whose
+    FP8Tensor always scales from the current tensor (src/nanotron/fp8/tensor.py:25-28).
+
+    The first quantisation through a fresh state (no finite positive amax recorded yet) uses
+    current scaling, exactly the reference's behaviour; from then on every step is a single
+    fused pass: cast with the held scale, amax, history roll, next scale."""
+
+    def __init__(self, dtype: DTypes, history_len: int = DEFAULT_AMAX_HISTORY_LEN, margin: int = DEFAULT_MARGIN,
+                 device: Union[str, torch.device] = "cuda"):
+        assert isinstance(dtype, DTypes) and dtype in _FMT
+        assert history_len >= 1
+        self.dtype = dtype
+        self.margin = _int_margin(margin)
+        self.history_len = int(history_len)
+        # one allocation: [scale, hist[0..H-1]]
+        self._buf = torch.zeros(1 + self.history_len, dtype=torch.float32, device=device)
+        self._buf[0] = INITIAL_SCALING_FACTOR
+        self.initialised = False
+
+    @property
+    def scale(self) -> torch.Tensor:
+        return self._buf[0]
+
+    @property
+    def amax_history(self) -> torch.Tensor:
+        return self._buf[1:]
+
+    def state_dict(self):
+        return {"buf": self._buf.clone(), "initialised": self.initialised}
+
+    def load_state_dict(self, sd):
+        self._buf.copy_(sd["buf"])
+        self.initialised = bool(sd["initialised"])
+
+
+class FP8Tensor(torch.Tensor):
+    """uint8 tensor holding OCP fp8 bytes plus `fp8_meta` (reference: src/nanotron/fp8/tensor.py:9-36).
+
+    `FP8Tensor(tensor, dtype)` is the reference call (current scaling).  Keyword-only extensions:
+    `state` selects delayed scaling for a tensor role, `with_transpose` also produces the
+    transposed bytes in the same pass (what the backward GEMMs consume)."""
+
+    def __new__(cls, tensor: torch.Tensor, dtype: DTypes, *, state: Optional[DelayedScaling] = None,
+                with_transpose: bool = False, margin: int = 0) -> "FP8Tensor":
+        assert isinstance(tensor, torch.Tensor), "tensor must be a tensor"
+        assert tensor.dtype not in FP8_DTYPES, "The tensor already quantized to FP8"
+        assert tensor.device != torch.device("cpu"), "FP8Tensor only supports CUDA device"
+        assert isinstance(dtype, DTypes)
+        return _quantize(cls, tensor, dtype, state, with_transpose, margin)
+
+    def transposed(self) -> "FP8Tensor":
+        """The [cols, rows] bytes as an FP8Tensor sharing this tensor's meta (reference:
+        tex.fp8_transpose, src/nanotron/fp8/kernel.py:43-44).  Cached."""
+        t = getattr(self, "_transposed", None)
+        if t is None:
+            assert self.dim() == 2, "transposed() needs a 2-D FP8Tensor"
+            rows, cols = self.shape
+            out = torch.empty((cols, rows), dtype=torch.uint8, device=self.device)
+            src = self if self.is_contiguous() else self.contiguous()
+            nt.check(nt.lib.ntfp8_transpose(src.data_ptr(), rows, cols, out.data_ptr(), nt.stream_ptr(self.device)),
+                     "ntfp8_transpose")
+            t = torch.Tensor._make_subclass(FP8Tensor, out)
+            t.fp8_meta = self.fp8_meta
+            self._transposed = t
+        return t
+
+    def __repr__(self) -> str:
+        return f"FP8Tensor({self.as_subclass(torch.Tensor)}, fp8_meta={self.fp8_meta})"
+
+
+def _quantize(cls, tensor: torch.Tensor, dtype: DTypes, state: Optional[DelayedScaling], with_transpose: bool,
+              margin: int = 0) -> FP8Tensor:
+    from nanotron_amd.fp8.meta import FP8Meta
+
+    if dtype not in _FMT:
+        raise ValueError(f"{dtype} is not an FP8 format")
+    if tensor.dtype not in nt.TORCH_TO_NT:
+        raise TypeError(f"cannot quantise a {tensor.dtype} tensor to FP8 (float32 / float16 / bfloat16 only)")
+    if tensor.numel() == 0:
+        raise RuntimeError("cannot quantise an empty tensor (amax of an empty tensor is undefined)")
+    x = tensor.detach()
+    if not x.is_contiguous():
+        x = x.contiguous()
+    dev = x.device
+    if x.dim() >= 2:
+        cols = x.shape[-1]
+        rows = x.numel() // cols
+    else:
+        rows, cols = 1, x.numel()
+    out = torch.empty(x.shape, dtype=torch.uint8, device=dev)
+    out_t = None
+    if with_transpose:
+        assert x.dim() == 2, "with_transpose needs a 2-D tensor"
+        out_t = torch.empty((cols, rows), dtype=torch.uint8, device=dev)
+    scalars = torch.empty(2, dtype=torch.float32, device=dev)  # [amax, scale used]
+    amax, scale = scalars[0], scalars[1]
+    ws = nt.workspace(dev)
+    st = nt.stream_ptr(dev)
+    fmt = _FMT[dtype]
+    xd = nt.TORCH_TO_NT[x.dtype]
+    if state is None:
+        nt.check(nt.lib.ntfp8_quantize_current(x.data_ptr(), xd, rows, cols, fmt, _int_margin(margin), amax.data_ptr(),
+                                               scale.data_ptr(), out.data_ptr(), nt.ptr(out_t), None, 0, None,
+                                               ws.data_ptr(), st), "ntfp8_quantize_current")
+    else:
+        assert state.dtype == dtype, "delayed-scaling state was created for another format"
+        assert state._buf.device == dev
+        if not state.initialised:
+            nt.check(nt.lib.ntfp8_quantize_current(x.data_ptr(), xd, rows, cols, fmt, state.margin, amax.data_ptr(),
+                                                   scale.data_ptr(), out.data_ptr(), nt.ptr(out_t),
+                                                   state.amax_history.data_ptr(), state.history_len,
+                                                   state.scale.data_ptr(), ws.data_ptr(), st),
+                     "ntfp8_quantize_current")
+            # only while the role has never seen a usable amax: one host read to learn whether it has now
+            a = float(amax.item())
+            state.initialised = a > 0.0 and a != float("inf")
+        else:
+            nt.check(nt.lib.ntfp8_quantize_delayed(x.data_ptr(), xd, rows, cols, fmt, state.margin,
+                                                   state.scale.data_ptr(), state.amax_history.data_ptr(),
+                                                   state.history_len, amax.data_ptr(), scale.data_ptr(),
+                                                   out.data_ptr(), nt.ptr(out_t), ws.data_ptr(), st),
+                     "ntfp8_quantize_delayed")
+    meta = FP8Meta(amax, scale, dtype)
+    obj = torch.Tensor._make_subclass(cls, out)
+    obj.fp8_meta = meta
+    if out_t is not None:
+        t = torch.Tensor._make_subclass(FP8Tensor, out_t)
+        t.fp8_meta = meta
+        obj._transposed = t
+    return obj
+
+
+def convert_torch_dtype_to_te_dtype(dtype) -> DType:
+    """Reference: src/nanotron/fp8/tensor.py:39-55 (same key set, returns this library's enum)."""
+    mapping = {
+        torch.int32: "kInt32",
+        torch.float32: "kFloat32",
+        torch.float16: "kFloat16",
+        torch.bfloat16: "kBFloat16",
+        DTypes.FP8E4M3: "kFloat8E4M3",
+        DTypes.FP8E5M2: "kFloat8E5M2",
+        DTypes.KFLOAT16: "kFloat16",
+    }
+    return getattr(DType, mapping[dtype])
+
+
+def convert_tensor_to_fp8(tensor: torch.Tensor, meta) -> torch.Tensor:
+    """Cast with the scale held in `meta` (reference: src/nanotron/fp8/tensor.py:60-65,
+    tex.cast_to_fp8).  Returns the uint8 bytes.  meta.amax is left untouched: at the reference's
+    only call site it already equals max|x| (tensor.py:25-28), so TE's amax update is a no-op."""
+    assert tensor.device != torch.device("cpu"), "convert_tensor_to_fp8 only supports CUDA tensors"
+    x = tensor.detach().contiguous()
+    dev = x.device
+    scale = meta.scale
+    if not (isinstance(scale, torch.Tensor) and scale.device == dev and scale.dtype == torch.float32):
+        scale = torch.as_tensor(scale, dtype=torch.float32).to(dev)
+    scale = scale.reshape(())
+    cols = x.shape[-1] if x.dim() >= 2 else x.numel()
+    rows = x.numel() // cols
+    out = torch.empty(x.shape, dtype=torch.uint8, device=dev)
+    nt.check(nt.lib.ntfp8_cast_to_fp8(x.data_ptr(), nt.TORCH_TO_NT[x.dtype], rows, cols, scale.data_ptr(),
+                                      _FMT[meta.dtype], out.data_ptr(), None, nt.stream_ptr(dev)), "ntfp8_cast_to_fp8")
+    return out
+
+
+def convert_tensor_from_fp8(tensor: torch.Tensor, meta, dtype: torch.dtype) -> torch.Tensor:
+    """Dequantise (reference: src/nanotron/fp8/tensor.py:68-74, tex.cast_from_fp8)."""
+    assert isinstance(tensor, torch.Tensor)
+    assert isinstance(dtype, torch.dtype)
+    assert tensor.device != torch.device("cpu"), "convert_tensor_from_fp8 only supports CUDA tensors"
+    if dtype not in nt.TORCH_TO_NT:
+        raise TypeError(f"unsupported output dtype {dtype}")
+    q = tensor.as_subclass(torch.Tensor) if isinstance(tensor, FP8Tensor) else tensor
+    q = q.contiguous()
+    dev = q.device
+    scale = meta.scale
+    if not (isinstance(scale, torch.Tensor) and scale.device == dev and scale.dtype == torch.float32):
+        scale = torch.as_tensor(scale, dtype=torch.float32).to(dev)
+    out = torch.empty(q.shape, dtype=dtype, device=dev)
+    if q.numel():
+        nt.check(nt.lib.ntfp8_cast_from_fp8(q.data_ptr(), _FMT[meta.dtype], scale.data_ptr(), q.numel(), out.data_ptr(),
+                                            nt.TORCH_TO_NT[dtype], nt.stream_ptr(dev)), "ntfp8_cast_from_fp8")
+    return out
+
+
+def update_scaling_factor(amax: torch.Tensor, scaling_factor: torch.Tensor, dtype: DTypes,
+                          margin: float = 0) -> torch.Tensor:
+    """Power-of-two scale from an amax (reference: src/nanotron/fp8/tensor.py:77-105).
+
+    Device tensors are processed by the HIP kernel and the result stays on the device; when both
+    arguments are host tensors (as in FP8Linear.__init__, src/nanotron/fp8/linear.py:33-42) the
+    native library evaluates the same function on the host."""
+    assert amax.dtype == torch.float32
+    assert scaling_factor.dtype == torch.float32
+    fmt = _FMT[dtype]
+    m = _int_margin(margin)
+    if not amax.is_cuda and not scaling_factor.is_cuda:
+        a, s = torch.broadcast_tensors(amax, scaling_factor)
+        flat = [nt.update_scaling_factor_host(float(x), float(y), fmt, m)
+                for x, y in zip(a.reshape(-1).tolist(), s.reshape(-1).tolist())]
+        return torch.tensor(flat, dtype=torch.float32).reshape(a.shape)
+    dev = amax.device if amax.is_cuda else scaling_factor.device
+    a, s = torch.broadcast_tensors(amax.to(dev), scaling_factor.to(dev))
+    a, s = a.contiguous(), s.contiguous()
+    out = torch.empty_like(a)
+    if a.numel():
+        nt.check(nt.lib.ntfp8_update_scaling_factor(a.data_ptr(), s.data_ptr(), fmt, m, out.data_ptr(), a.numel(),
+                                                    nt.stream_ptr(dev)), "ntfp8_update_scaling_factor")
+    return out

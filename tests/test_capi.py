@@ -1,0 +1,142 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every symbol the header declares, the
+Python binding covers all of them, and argument errors are reported as codes before any launch."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ntfp8.h")
+
+
+def declared_functions():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(ntfp8_[a-z0-9_]+)\s*\(", src)))
+
+
+def test_library_exports_every_declared_symbol():
+    from nanotron_amd import _native as nt
+
+    names = declared_functions()
+    assert len(names) >= 11
+    for n in names:
+        assert hasattr(nt.lib, n), f"{n} declared in include/ntfp8.h but not exported"
+        assert n in nt.SIGNATURES, f"{n} has no ctypes signature"
+    assert sorted(nt.SIGNATURES) == names
+    assert nt.version() == 1
+    assert nt.strerror(0) == "ok" and "NULL" in nt.strerror(-1)
+
+
+def test_header_constants_match_binding():
+    from nanotron_amd import _native as nt
+
+    src = open(HEADER).read()
+    assert int(re.search(r"#define NTFP8_WORKSPACE_BYTES (\d+)", src).group(1)) == nt.WORKSPACE_BYTES
+    assert re.search(r"NTFP8_E4M3 = 0, NTFP8_E5M2 = 1", src)
+    assert re.search(r"NTFP8_F32 = 0, NTFP8_F16 = 1, NTFP8_BF16 = 2", src)
+
+
+def test_argument_errors_are_codes_not_faults():
+    from nanotron_amd import _native as nt
+
+    L = nt.lib
+    P = 0x10000  # a non-NULL, 16-byte aligned fake pointer: never dereferenced when validation fails
+    # NULL pointers
+    assert L.ntfp8_gemm(None, 0, P, P, 0, P, P, 0, 16, 16, 16, 0, None) == -1
+    assert L.ntfp8_cast_to_fp8(None, 2, 4, 4, P, 0, P, None, None) == -1
+    assert L.ntfp8_cast_to_fp8(P, 2, 4, 4, P, 0, None, None, None) == -1
+    assert L.ntfp8_quantize_delayed(P, 2, 4, 4, 0, 0, None, P, 16, P, P, P, None, P, None) == -1
+    assert L.ntfp8_amax_scale(P, 2, 16, 0, 0, None, None, P, P, None) == -1
+    assert L.ntfp8_transpose(None, 4, 4, P, None) == -1
+    assert L.ntfp8_cast_from_fp8(P, 0, None, 16, P + 4096, 0, None) == -1
+    # bad enums
+    assert L.ntfp8_gemm(P, 7, P, P, 0, P, P + (1 << 20), 0, 16, 16, 16, 0, None) == -2
+    assert L.ntfp8_cast_to_fp8(P, 9, 4, 4, P, 0, P + 4096, None, None) == -2
+    assert L.ntfp8_cast_from_fp8(P, 0, P, 16, P + 4096, 5, None) == -2
+    # sizes
+    assert L.ntfp8_gemm(P, 0, P, P, 0, P, P + (1 << 20), 0, 0, 16, 16, 0, None) == -3
+    assert L.ntfp8_gemm(P, 0, P, P, 0, P, P + (1 << 20), 0, 16, -1, 16, 0, None) == -3
+    assert L.ntfp8_cast_to_fp8(P, 2, 0, 4, P, 0, P + 4096, None, None) == -3
+    assert L.ntfp8_cast_to_fp8(P, 2, 1 << 40, 1 << 40, P, 0, P + 4096, None, None) == -3
+    assert L.ntfp8_quantize_delayed(P, 2, 4, 4, 0, 0, P, P, 0, P, P, P + 4096, None, P, None) == -3
+    assert L.ntfp8_quantize_delayed(P, 2, 4, 4, 0, 500, P, P, 16, P, P, P + 4096, None, P, None) == -3
+    assert L.ntfp8_amax_scale(P, 2, 0, 0, 0, None, P, P, P, None) == -3
+    # alignment
+    assert L.ntfp8_cast_to_fp8(P + 1, 2, 4, 4, P, 0, P + 4096, None, None) == -4
+    assert L.ntfp8_cast_to_fp8(P, 0, 4, 4, P + 2, 0, P + 4096, None, None) == -4
+    assert L.ntfp8_gemm(P, 0, P + 1, P, 0, P, P + (1 << 20), 0, 16, 16, 16, 0, None) == -4
+    # unsupported: accumulate into a 16-bit output
+    assert L.ntfp8_gemm(P, 0, P, P + 4096, 0, P, P + (1 << 20), 2, 16, 16, 16, 1, None) == -5
+    # aliasing
+    assert L.ntfp8_cast_to_fp8(P, 2, 4, 4, P + 4096, 0, P + 8, None, None) == -7
+    assert L.ntfp8_transpose(P, 4, 4, P + 8, None) == -7
+    assert L.ntfp8_gemm(P, 0, P + 4096, P + 8192, 0, P + 4096, P + 64, 0, 16, 16, 16, 0, None) == -7
+
+
+def test_host_scale_function_matches_oracle():
+    from nanotron_amd import _native as nt
+    from oracle import fp8_oracle as O
+
+    f32 = lambda v: torch.tensor(v, dtype=torch.float32)
+    for fmt, f in ((O.E4M3, nt.E4M3), (O.E5M2, nt.E5M2)):
+        assert nt.update_scaling_factor_host(1.0, 1.0, f, 0) == (256.0 if fmt == O.E4M3 else 32768.0)
+        bits = torch.arange(1, 0x7F80, 7, dtype=torch.int32).to(torch.int16)
+        vals = bits.view(torch.bfloat16).float()
+        want = O.update_scaling_factor(vals, torch.ones_like(vals), fmt)
+        got = [nt.update_scaling_factor_host(v, 1.0, f, 0) for v in vals.tolist()]
+        assert got == want.tolist()
+        for a in (0.0, -2.0, float("nan"), float("inf"), 1e-38, 3e38):
+            for m in (0, 2):
+                w = O.update_scaling_factor(f32(a), f32(3.0), fmt, m).item()
+                assert nt.update_scaling_factor_host(a, 3.0, f, m) == w, (a, m)
+        # quotients a few ulps around powers of two
+        ks = torch.arange(-20, 21, dtype=torch.float32)
+        p = torch.pow(torch.tensor(2.0), ks)
+        for d in (-2, -1, 0, 1):
+            a = torch.tensor(O.FP8_MAX[fmt]) / (p.view(torch.int32) + d).view(torch.float32)
+            w = O.update_scaling_factor(a, torch.ones_like(a), fmt).tolist()
+            assert [nt.update_scaling_factor_host(v, 1.0, f, 0) for v in a.tolist()] == w
+
+
+def test_python_api_surface_matches_reference_names():
+    import nanotron_amd
+    from nanotron_amd.fp8 import DTypes, FP8Linear, FP8Parameter, FP8Tensor  # noqa: F401
+    from nanotron_amd.fp8.constants import DTYPE_TO_FP8_MAX, FP8_DTYPES, INITIAL_AMAX, INITIAL_SCALING_FACTOR
+    from nanotron_amd.fp8.kernel import fp8_matmul_kernel  # noqa: F401
+    from nanotron_amd.fp8.meta import FP8Meta
+    from nanotron_amd.fp8.tensor import (convert_tensor_from_fp8, convert_tensor_to_fp8,  # noqa: F401
+                                         convert_torch_dtype_to_te_dtype, update_scaling_factor)
+    from nanotron_amd.fp8.utils import is_fp8_available
+
+    assert [d.name for d in DTypes] == ["FP8E4M3", "FP8E5M2", "KFLOAT16"]
+    assert DTYPE_TO_FP8_MAX[DTypes.FP8E4M3] == 448.0 and DTYPE_TO_FP8_MAX[DTypes.FP8E5M2] == 57344.0
+    assert INITIAL_AMAX == 1.0 and INITIAL_SCALING_FACTOR == 1.0 and torch.uint8 in FP8_DTYPES
+    assert convert_torch_dtype_to_te_dtype(DTypes.FP8E4M3).name == "kFloat8E4M3"
+    assert convert_torch_dtype_to_te_dtype(torch.bfloat16).name == "kBFloat16"
+    # update_scaling_factor on host tensors (what FP8Linear.__init__ evaluates, linear.py:33-42)
+    s = update_scaling_factor(torch.tensor(1.0), torch.tensor(1.0), DTypes.FP8E4M3)
+    assert s.item() == 256.0 and s.dtype == torch.float32
+    assert update_scaling_factor(torch.tensor(1.0), torch.tensor(1.0), DTypes.FP8E5M2).item() == 32768.0
+    with pytest.raises(ValueError):
+        update_scaling_factor(torch.tensor(1.0), torch.tensor(1.0), DTypes.FP8E4M3, margin=0.5)
+    m = FP8Meta(torch.tensor(2.0), torch.tensor(4.0), DTypes.FP8E4M3)
+    assert m.fp8_max == 448.0 and m.inverse_scale.item() == 0.25 and m.te_dtype.name == "kFloat8E4M3"
+    assert isinstance(is_fp8_available(), bool)
+    # CPU construction keeps a plain nn.Parameter and falls back to F.linear (linear.py:28,53-54)
+    lin = FP8Linear(8, 4, device="cpu")
+    assert type(lin.weight) is torch.nn.Parameter
+    x = torch.randn(3, 8, requires_grad=True)
+    lin(x).sum().backward()
+    assert lin.weight.grad.shape == (4, 8) and x.grad is not None
+    with pytest.raises(AssertionError):
+        FP8Tensor(torch.randn(4, 4), DTypes.FP8E4M3)  # CPU tensors are rejected (tensor.py:22)
+    with pytest.raises(AssertionError):
+        FP8Parameter(torch.randn(4, 4), DTypes.FP8E4M3)
+    nanotron_amd.install_as_nanotron_fp8()
+    from nanotron.fp8 import FP8Linear as RefPathLinear  # noqa
+    from nanotron.fp8.tensor import update_scaling_factor as ref_path_usf  # noqa
+
+    assert RefPathLinear is FP8Linear
