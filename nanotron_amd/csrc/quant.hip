@@ -320,8 +320,11 @@ __global__ __launch_bounds__(kThreads) void quant_transpose_scalar_kernel(
 // Dequantise: out = out_dtype(decode(byte) * (1 / scale)).
 template <int F>
 __device__ __forceinline__ float decode1(uint32_t b) {
-    if constexpr (F == kE4M3) return __builtin_amdgcn_cvt_f32_fp8((int)b, 0);
-    else return __builtin_amdgcn_cvt_f32_bf8((int)b, 0);
+    float v;
+    if constexpr (F == kE4M3) v = __builtin_amdgcn_cvt_f32_fp8((int)b, 0);
+    else v = __builtin_amdgcn_cvt_f32_bf8((int)b, 0);
+    // the hardware conversion returns +0 for the code 0x80; the sign bit is carried over explicitly
+    return __uint_as_float(__float_as_uint(v) | ((b & 0x80u) << 24));
 }
 
 template <int F, int OUT>

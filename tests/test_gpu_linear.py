@@ -50,9 +50,21 @@ def test_fp8_linear_backward_pass(input_requires_grad, device):
     fp8_linear.bias.data = ref_linear.bias.detach().clone()
     ref_linear(ref_input).sum().backward()
     fp8_linear(input).sum().backward()
-    assert torch.allclose(fp8_linear.weight.grad, ref_linear.weight.grad, 0.1, 0.1)
     assert torch.allclose(fp8_linear.bias.grad, ref_linear.bias.grad, 0, 0.1)
+    if device == "cpu":
+        assert torch.allclose(fp8_linear.weight.grad, ref_linear.weight.grad, 0.1, 0.1)
+        return
+    # Against the un-quantised fp32 layer the reference asserts rtol=atol=0.1.  Each e4m3 input carries
+    # up to 2^-4 relative rounding error and dW sums 16 of them, so that bound is itself noisy (the
+    # reference never runs this test in CI); here it is asserted against the oracle, which computes
+    # the same quantised arithmetic, and only loosely against the fp32 layer.
+    xq = O.quantise_current(ref_input.detach().cpu(), O.E4M3)
+    wq = O.quantise_current(ref_linear.weight.detach().cpu(), O.E4M3)
+    gq = O.quantise_current(torch.ones(16, 16), O.E5M2)
+    assert torch.allclose(fp8_linear.weight.grad.cpu(), O.linear_wgrad(gq, xq), 1e-3, 1e-3)
+    assert torch.allclose(fp8_linear.weight.grad, ref_linear.weight.grad, 0.1, 0.5)
     if input_requires_grad:
+        assert torch.allclose(input.grad.cpu(), O.linear_dgrad(gq, wq), 1e-3, 1e-3)
         assert torch.allclose(input.grad, ref_input.grad, 0.1, 0.1)
 
 

@@ -251,7 +251,10 @@ def test_delayed_scaling_zero_first_then_values(fmt):
         assert got.fp8_meta.scale.item() == want.scale.item(), i
         assert st.scale.item() == ref.scale.item(), i
         assert torch.equal(st.amax_history.cpu(), ref.hist), i
-        assert torch.equal(got.cpu().as_subclass(torch.Tensor), want.q), i
+        q = got.cpu().as_subclass(torch.Tensor)
+        assert torch.equal(q, want.q), i
+        if i in (2, 6):  # 900.0 cast with the stale scale of the 2.0 step: clipped to +max
+            assert int(q[0, 0]) == (0x7E if fmt == O.E4M3 else 0x7B)
 
 
 @pytest.mark.parametrize("fmt", FMTS)
@@ -260,7 +263,6 @@ def test_config2_full_size_20_steps(fmt):
     _, _, DelayedScaling, FP8Tensor, _ = _api()
     st = DelayedScaling(_dt(fmt), history_len=16)
     ref = O.DelayedScaling(fmt, history_len=16)
-    saturated = 0
     for step in range(20):
         x = O.student_t_outlier_tensor(1234 + 100 * 2 + step, (4096, 4096))
         want = ref.quantise(x)
@@ -271,8 +273,6 @@ def test_config2_full_size_20_steps(fmt):
         assert torch.equal(st.amax_history.cpu(), ref.hist), step
         q = got.cpu().as_subclass(torch.Tensor)
         assert torch.equal(q, want.q), step
-        saturated += int(((q & 0x7F) == (0x7E if fmt == O.E4M3 else 0x7B)).sum())
-    assert saturated > 0  # the stale scale really does clip outliers
 
 
 # ------------------------------------------------------------------ the reference's own tests, mirrored
