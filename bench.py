@@ -1,0 +1,312 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload linear|quant] [--no-cpu-baseline]
+
+Default workload ("linear"): the Llama-3-8B decoder-block linears of the benchmark configuration,
+forward + backward with delayed scaling (history 16, margin 0) at 4096 tokens:
+QKV 4096->6144, O 4096->4096, gate 4096->14336, up 4096->14336, down 14336->4096.
+One step = for every linear: re-quantise the weight (e4m3, + transpose), quantise the activation
+(e4m3, + transpose), forward GEMM (bf16 out), quantise the output gradient (e5m2, + transpose),
+dgrad GEMM (bf16 out), wgrad GEMM (fp32 out).  All inputs are resident in HBM before the timed
+region.  value = GEMM FLOPs of the step (6*M*N*K per linear) / wall time of the step, so the
+quantisation passes are inside the time but contribute no FLOPs.
+
+Workload "quant": benchmark configuration 2, the fused amax + history roll + scale update +
+saturating cast on bf16 [4096,4096], e4m3 and e5m2 alternating, 8 rotating input buffers.
+
+One JSON line is printed.  `roofline` describes the dominant kernel (the fp8 MFMA GEMM for
+"linear", the fused quantise kernel for "quant"), timed with events on the launch stream;
+`cpu_baseline` is the CPU oracle (a port of the reference's arithmetic) timed on this host.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA peak
+PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E peak
+
+TOKENS = 4096
+LINEARS = [  # name, in_features (K), out_features (N)
+    ("qkv", 4096, 6144),
+    ("o", 4096, 4096),
+    ("gate", 4096, 14336),
+    ("up", 4096, 14336),
+    ("down", 14336, 4096),
+]
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=20)
+    p.add_argument("--warmup", type=int, default=5)
+    p.add_argument("--workload", choices=["linear", "quant"], default="linear")
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--kernel-reps", type=int, default=20, help="launches per GEMM shape for the roofline timing")
+    return p.parse_args()
+
+
+def event_time_ms(fn, reps, warm=3):
+    import torch
+
+    for _ in range(warm):
+        fn()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(reps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / reps
+
+
+# ------------------------------------------------------------------------------------ linear workload
+def build_linears(device):
+    import torch
+
+    from nanotron_amd.fp8 import FP8Linear
+
+    g = torch.Generator(device="cpu").manual_seed(1234 + 500)
+    mods, xs, gys = [], [], []
+    for name, K, N in LINEARS:
+        lin = FP8Linear(K, N, bias=False, device=device, out_dtype=torch.bfloat16, delayed_scaling=True,
+                        amax_history_len=16, margin=0)
+        w = (torch.randn(N, K, generator=g, dtype=torch.float32) * 0.02)
+        with torch.no_grad():
+            lin.weight.as_subclass(torch.Tensor).copy_(w.to(device))
+        mods.append(lin)
+        xs.append((torch.randn(TOKENS, K, generator=g, dtype=torch.float32)).to(torch.bfloat16).to(device))
+        gys.append((torch.randn(TOKENS, N, generator=g, dtype=torch.float32) * 1e-3).to(torch.bfloat16).to(device))
+    return mods, xs, gys
+
+
+def linear_step(mods, xs, gys):
+    for lin, x, gy in zip(mods, xs, gys):
+        lin.requantize_weight()
+        x.grad = None
+        y = lin(x)
+        y.backward(gy)
+
+
+def gemm_roofline(mods, xs, gys, reps):
+    """Per-launch timing of the GEMM kernel on the shapes of the step (events on the launch stream)."""
+    import torch
+
+    from nanotron_amd.fp8 import DTypes, FP8Tensor
+    from nanotron_amd.fp8.kernel import _gemm_nt
+
+    total_flops, total_ms, per_shape = 0.0, 0.0, []
+    for (name, K, N), lin, x, gy in zip(LINEARS, mods, xs, gys):
+        xq = FP8Tensor(x.detach(), DTypes.FP8E4M3, with_transpose=True)
+        gq = FP8Tensor(gy, DTypes.FP8E5M2, with_transpose=True)
+        wq = lin.weight.data
+        calls = [
+            ("fwd", lambda: _gemm_nt(xq, wq, torch.bfloat16, None)),
+            ("dgrad", lambda: _gemm_nt(gq, wq.transposed(), torch.bfloat16, None)),
+            ("wgrad", lambda: _gemm_nt(gq.transposed(), xq.transposed(), torch.float32, None)),
+        ]
+        flops = 2.0 * TOKENS * N * K
+        for tag, fn in calls:
+            ms = event_time_ms(fn, reps)
+            total_flops += flops
+            total_ms += ms
+            per_shape.append({"gemm": f"{name}.{tag}", "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1)})
+    return total_flops, total_ms, per_shape
+
+
+def cpu_baseline_linear():
+    """The oracle's arithmetic for one linear (the O projection, 4096x4096x4096) forward + backward
+    on this host: amax/scale/cast of X, W, dY and the three fp32 GEMMs on exactly-upcast operands."""
+    import torch
+
+    from oracle import fp8_oracle as O
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    M = K = N = 4096
+    x = O.normal_tensor(1, (M, K), 1.0)
+    w = O.normal_tensor(2, (N, K), 0.02)
+    gy = O.normal_tensor(3, (M, N), 1e-3)
+
+    def run():
+        xq, wq, gq = O.quantise_current(x, O.E4M3), O.quantise_current(w, O.E4M3), O.quantise_current(gy, O.E5M2)
+        y = O.linear_forward(xq, wq, torch.bfloat16)
+        dx = O.linear_dgrad(gq, wq, torch.bfloat16)
+        dw = O.linear_wgrad(gq, xq)
+        return y, dx, dw
+
+    run()
+    t0 = time.perf_counter()
+    n = 0
+    while n < 2 or time.perf_counter() - t0 < 10.0:
+        run()
+        n += 1
+    dt = (time.perf_counter() - t0) / n
+    return {"value": round(6.0 * M * N * K / dt / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port", "sample": f"O projection 4096x4096x4096 fwd+bwd (quantise X,W,dY + 3 fp32 GEMMs), {n} runs"}
+
+
+# ------------------------------------------------------------------------------------ quant workload
+def build_quant(device, nbuf=8):
+    import torch
+
+    from nanotron_amd.fp8 import DelayedScaling, DTypes
+    from oracle import fp8_oracle as O
+
+    bufs = [O.student_t_outlier_tensor(1234 + 200 + i, (4096, 4096)).to(device) for i in range(nbuf)]
+    states = {DTypes.FP8E4M3: DelayedScaling(DTypes.FP8E4M3, 16, 0, device),
+              DTypes.FP8E5M2: DelayedScaling(DTypes.FP8E5M2, 16, 0, device)}
+    return bufs, states
+
+
+def quant_step(bufs, states, i):
+    from nanotron_amd.fp8 import FP8Tensor
+
+    x = bufs[i % len(bufs)]
+    for dt, st in states.items():
+        FP8Tensor(x, dt, state=st)
+
+
+def quant_kernel_ms(bufs, states, reps):
+    """Average duration of the fused delayed-scaling kernel alone (C ABI, preallocated outputs)."""
+    import torch
+
+    from nanotron_amd import _native as nt
+    from nanotron_amd.fp8 import DTypes
+
+    dev = bufs[0].device
+    out = [torch.empty(4096 * 4096, dtype=torch.uint8, device=dev) for _ in range(len(bufs))]
+    sc = torch.zeros(2, dtype=torch.float32, device=dev)
+    ws = nt.workspace(dev)
+    st = nt.stream_ptr(dev)
+    res = {}
+    for dt, fmt in ((DTypes.FP8E4M3, nt.E4M3), (DTypes.FP8E5M2, nt.E5M2)):
+        state = states[dt]
+        k = [0]
+
+        def fn():
+            i = k[0] % len(bufs)
+            k[0] += 1
+            nt.check(nt.lib.ntfp8_quantize_delayed(bufs[i].data_ptr(), nt.BF16, 4096, 4096, fmt, 0,
+                                                   state.scale.data_ptr(), state.amax_history.data_ptr(), 16,
+                                                   sc[0:].data_ptr(), sc[1:].data_ptr(), out[i].data_ptr(), None,
+                                                   ws.data_ptr(), st), "quantize_delayed")
+
+        res[dt.name] = event_time_ms(fn, reps, warm=8)
+    return res
+
+
+def cpu_baseline_quant():
+    import torch
+
+    from oracle import fp8_oracle as O
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    x = O.student_t_outlier_tensor(1234 + 200, (4096, 4096))
+    sts = [O.DelayedScaling(O.E4M3), O.DelayedScaling(O.E5M2)]
+    for s in sts:
+        s.quantise(x)
+    t0 = time.perf_counter()
+    n = 0
+    while n < 2 or time.perf_counter() - t0 < 10.0:
+        for s in sts:
+            s.quantise(x)
+        n += 1
+    dt = (time.perf_counter() - t0) / (2 * n)
+    return {"value": round(3.0 * x.numel() / dt / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port", "sample": f"bf16 [4096,4096] delayed-scaling quantise (amax, cast, roll), {2 * n} tensor-steps"}
+
+
+# ------------------------------------------------------------------------------------ main
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this hot path has no collectives and every box here has one GPU; "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (cuda:0)", file=sys.stderr)
+        sys.exit(2)
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+
+    if args.workload == "linear":
+        mods, xs, gys = build_linears(device)
+        xs = [x.requires_grad_(True) for x in xs]
+        step = lambda i: linear_step(mods, xs, gys)
+        flops_step = sum(6.0 * TOKENS * N * K for _, K, N in LINEARS)
+    else:
+        bufs, states = build_quant(device)
+        step = lambda i: quant_step(bufs, states, i)
+        bytes_step = 2 * 3.0 * 4096 * 4096
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(args.warmup + i)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+
+    out = {
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "data": "synthetic",
+    }
+    if args.workload == "linear":
+        value = flops_step / (ms_per_step * 1e-3) / 1e12
+        gf, gms, per_shape = gemm_roofline(mods, xs, gys, args.kernel_reps)
+        achieved = gf / (gms * 1e-3) / 1e12
+        out.update({
+            "metric": "FP8Linear fwd+bwd TFLOP/s", "value": round(value, 2), "unit": "TFLOP/s", "dtype": "fp8",
+            "config": {"workload": "llama3-8b decoder-block linears fwd+bwd, 4096 tokens, delayed scaling hist 16",
+                       "tokens": TOKENS, "linears": [f"{n}:{k}->{o}" for n, k, o in LINEARS],
+                       "flops_per_step": flops_step, "pct_fp8_peak": round(100 * value / PEAK_FP8_TFLOPS, 2)},
+            "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(achieved / PEAK_FP8_TFLOPS, 4), "traffic": None,
+                         "kernel": "gemm_nt_kernel", "launches": per_shape},
+        })
+        # secondary figure of the metric: the fused quantise kernel on configuration 2
+        bufs, states = build_quant(device)
+        qms = quant_kernel_ms(bufs, states, 64)
+        qb = 3.0 * 4096 * 4096
+        q_avg = sum(qms.values()) / len(qms)
+        out["quant"] = {"metric": "amax+quant GB/s", "value": round(qb / (q_avg * 1e-3) / 1e9, 1), "unit": "GB/s",
+                        "workload": "bf16 [4096,4096] fused amax+roll+scale+cast, 8 rotating buffers",
+                        "ms": {k: round(v, 5) for k, v in qms.items()},
+                        "roofline": {"bound": "hbm", "achieved": round(qb / (q_avg * 1e-3) / 1e9, 1),
+                                     "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                                     "frac": round(qb / (q_avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4), "traffic": None}}
+        if not args.no_cpu_baseline:
+            out["cpu_baseline"] = cpu_baseline_linear()
+    else:
+        value = bytes_step / (ms_per_step * 1e-3) / 1e9
+        qms = quant_kernel_ms(bufs, states, 64)
+        qb = 3.0 * 4096 * 4096
+        q_avg = sum(qms.values()) / len(qms)
+        out.update({
+            "metric": "amax+quant GB/s", "value": round(value, 1), "unit": "GB/s", "dtype": "bf16->fp8",
+            "config": {"workload": "bf16 [4096,4096] delayed-scaling quantise, e4m3 + e5m2 per step, hist 16",
+                       "bytes_per_step": bytes_step, "pct_hbm_peak": round(100 * value / PEAK_HBM_GBPS, 2)},
+            "roofline": {"bound": "hbm", "achieved": round(qb / (q_avg * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBPS,
+                         "unit": "GB/s", "frac": round(qb / (q_avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4), "traffic": None,
+                         "kernel": "quant_flat_kernel", "ms": {k: round(v, 5) for k, v in qms.items()}},
+        })
+        if not args.no_cpu_baseline:
+            out["cpu_baseline"] = cpu_baseline_quant()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

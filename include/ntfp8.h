@@ -28,7 +28,7 @@ extern "C" {
 #endif
 
 #define NTFP8_VERSION 1
-#define NTFP8_WORKSPACE_BYTES 64
+#define NTFP8_WORKSPACE_BYTES 2048
 
 /* FP8 storage formats.  Reference: DTypes.FP8E4M3 / DTypes.FP8E5M2 (src/nanotron/fp8/dtypes.py:4-7),
  * mapped to tex.DType.kFloat8E4M3 / kFloat8E5M2 at src/nanotron/fp8/tensor.py:39-55. */

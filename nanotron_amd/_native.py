@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libntfp8.so")
 
 E4M3, E5M2 = 0, 1
 F32, F16, BF16 = 0, 1, 2
-WORKSPACE_BYTES = 64
+WORKSPACE_BYTES = 2048
 
 TORCH_TO_NT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 

@@ -40,7 +40,10 @@ struct OutT<NTFP8_BF16> {
 template <>
 struct OutT<NTFP8_F16> {
     typedef uint16_t type;
-    __device__ static __forceinline__ uint16_t cvt(float v) { return __half_as_ushort(__float2half_rn(v)); }
+    __device__ static __forceinline__ uint16_t cvt(float v) {
+        asm volatile("" : "+v"(v));  // no folding of the descale multiply into a mixed-precision fma (-0 would become +0)
+        return __half_as_ushort(__float2half_rn(v));
+    }
 };
 
 template <int FA, int FB, int DT, bool kAcc>

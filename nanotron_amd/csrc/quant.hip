@@ -6,7 +6,9 @@
 
 namespace ntfp8 {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 256;       // dequant / transpose / scalar kernels
+constexpr int kFlatThreads = 1024;  // streaming quantise kernel: one block per CU, 16 waves
+constexpr int kTileThreads = 256;   // tile (transposing) quantise kernel
 constexpr int kVec = 16;  // elements per thread per step: 16 fp8 bytes = one 128-bit store
 
 typedef float f4 __attribute__((ext_vector_type(4)));
@@ -133,8 +135,14 @@ __device__ __forceinline__ uint8_t encode1(float x, float scale) {
 
 // ---------------------------------------------------------------------------------------------
 // Block reduction of the partial max, publication, and the last-block epilogue.
+//
+// Inter-block traffic uses relaxed device-scope atomics only (they execute at the level where all
+// XCDs agree) and orders them with the wave's own memory counter: the partial max is folded in with
+// a returning atomic, the wave waits for it, then takes a ticket.  A release fence here would write
+// back the whole L2 once per block, which costs more than the streaming pass itself.
+template <int THREADS>
 __device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, const ScalarIO& io, int mode) {
-    __shared__ uint32_t s_part[kThreads / 64];
+    __shared__ uint32_t s_part[THREADS / 64];
     __shared__ bool s_last;
     const uint32_t wm = wave_max_u32(m_f32bits);
     if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = wm;
@@ -142,16 +150,21 @@ __device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, c
     if (threadIdx.x == 0) {
         uint32_t bm = 0;
 #pragma unroll
-        for (int i = 0; i < kThreads / 64; ++i) bm = s_part[i] > bm ? s_part[i] : bm;
-        if (bm) __hip_atomic_fetch_max(&ws->amax_bits, bm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __threadfence();
-        const uint32_t t = __hip_atomic_fetch_add(&ws->ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        for (int i = 0; i < THREADS / 64; ++i) bm = s_part[i] > bm ? s_part[i] : bm;
+        const uint32_t old = __hip_atomic_fetch_max(&ws->slot[blockIdx.x % kMaxSlots].bits, bm, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::"v"(old) : "memory");
+        const uint32_t t = __hip_atomic_fetch_add(&ws->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_last = (t == gridDim.x - 1);
     }
     __syncthreads();
     if (!s_last || threadIdx.x != 0) return;
-    __threadfence();
-    uint32_t bits = __hip_atomic_load(&ws->amax_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t bits = 0;
+#pragma unroll
+    for (int i = 0; i < kMaxSlots; ++i) {
+        const uint32_t v = __hip_atomic_load(&ws->slot[i].bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        bits = v > bits ? v : bits;
+    }
     if (bits > kInfBits) bits = kNanBits;
     const float a = __uint_as_float(bits);
     *io.amax_out = a;
@@ -175,8 +188,10 @@ __device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, c
         if (hm > kInfBits) hm = kNanBits;
         *io.scale_state = update_scale(__uint_as_float(hm), used, io.fmt, io.margin);
     }
-    __hip_atomic_store(&ws->amax_bits, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&ws->ticket, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int i = 0; i < kMaxSlots; ++i)
+        __hip_atomic_store(&ws->slot[i].bits, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&ws->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ bool degenerate_scale(float s) {
@@ -187,7 +202,7 @@ __device__ __forceinline__ bool degenerate_scale(float s) {
 // ---------------------------------------------------------------------------------------------
 // Flat (no transpose) kernel: amax only, cast only, or both (delayed scaling).
 template <typename S, int F, int MODE>
-__global__ __launch_bounds__(kThreads) void quant_flat_kernel(const typename ElemOf<S>::type* __restrict__ x,
+__global__ __launch_bounds__(kFlatThreads) void quant_flat_kernel(const typename ElemOf<S>::type* __restrict__ x,
                                                               int64_t n_vec, int64_t n, uint8_t* __restrict__ out,
                                                               const float* __restrict__ scale_ptr, Workspace* ws,
                                                               ScalarIO io) {
@@ -201,8 +216,8 @@ __global__ __launch_bounds__(kThreads) void quant_flat_kernel(const typename Ele
         degen = degenerate_scale(scale);
     }
     uint32_t m_run = 0;  // in source-format bits
-    const int64_t stride = (int64_t)gridDim.x * kThreads;
-    int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * kFlatThreads;
+    int64_t i = (int64_t)blockIdx.x * kFlatThreads + threadIdx.x;
     // two groups per trip: four (bf16) or eight (fp32) 128-bit loads in flight per lane
     for (; i + stride < n_vec; i += 2 * stride) {
         float v0[16], v1[16];
@@ -231,13 +246,13 @@ __global__ __launch_bounds__(kThreads) void quant_flat_kernel(const typename Ele
         }
     }
     // elements the vector body does not cover (tail, or everything when a pointer is misaligned)
-    for (int64_t j = n_vec * kVec + (int64_t)blockIdx.x * kThreads + threadIdx.x; j < n; j += stride) {
+    for (int64_t j = n_vec * kVec + (int64_t)blockIdx.x * kFlatThreads + threadIdx.x; j < n; j += stride) {
         uint32_t m;
         const float xv = L::load1(x + j, m);
         if constexpr (kAmax) m_run = m > m_run ? m : m_run;
         if constexpr (kCast) out[j] = encode1<F>(xv, scale);
     }
-    if constexpr (kAmax) publish_and_finalize(L::to_f32_bits(m_run), ws, io, MODE);
+    if constexpr (kAmax) publish_and_finalize<kFlatThreads>(L::to_f32_bits(m_run), ws, io, MODE);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -248,7 +263,7 @@ __global__ __launch_bounds__(kThreads) void quant_flat_kernel(const typename Ele
 constexpr int kTile = 128;
 
 template <typename S, int F, bool kAmax>
-__global__ __launch_bounds__(kThreads) void quant_transpose_kernel(const typename ElemOf<S>::type* __restrict__ x,
+__global__ __launch_bounds__(kTileThreads) void quant_transpose_kernel(const typename ElemOf<S>::type* __restrict__ x,
                                                                    int64_t rows, int64_t cols,
                                                                    uint8_t* __restrict__ out,
                                                                    uint8_t* __restrict__ out_t,
@@ -259,12 +274,15 @@ __global__ __launch_bounds__(kThreads) void quant_transpose_kernel(const typenam
     const float scale = *scale_ptr;
     const bool degen = degenerate_scale(scale);
     const int64_t tiles_c = cols / kTile;
-    const int64_t tr = blockIdx.x / tiles_c, tc = blockIdx.x % tiles_c;
-    const int64_t row0 = tr * kTile, col0 = tc * kTile;
+    const int64_t tiles = (rows / kTile) * tiles_c;
     const int t = threadIdx.x;
     const int cchunk = t & 7;   // 16-column chunk inside the tile
     const int rsub = t >> 3;    // 0..31
+    const int rchunk = t & 7;
     uint32_t m_run = 0;
+    // persistent over tiles: the number of blocks (and so of reduction atomics) stays ~2 per CU
+    for (int64_t tile_id = blockIdx.x; tile_id < tiles; tile_id += gridDim.x) {
+    const int64_t row0 = (tile_id / tiles_c) * kTile, col0 = (tile_id % tiles_c) * kTile;
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
         const int r = rsub + 32 * it;
@@ -282,7 +300,6 @@ __global__ __launch_bounds__(kThreads) void quant_transpose_kernel(const typenam
             tile[(cchunk * 16 + j) * kTile + rsw] = (uint8_t)(w[j >> 2] >> (8 * (j & 3)));
     }
     __syncthreads();
-    const int rchunk = t & 7;
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
         const int c = rsub + 32 * it;
@@ -290,7 +307,9 @@ __global__ __launch_bounds__(kThreads) void quant_transpose_kernel(const typenam
         const u4 q = *reinterpret_cast<const u4*>(&tile[c * kTile + pos]);
         __builtin_nontemporal_store(q, reinterpret_cast<u4*>(out_t + (col0 + c) * rows + row0 + rchunk * 16));
     }
-    if constexpr (kAmax) publish_and_finalize(L::to_f32_bits(m_run), ws, io, kModeDelayed);
+    __syncthreads();  // the tile buffer is reused by the next trip
+    }
+    if constexpr (kAmax) publish_and_finalize<kTileThreads>(L::to_f32_bits(m_run), ws, io, kModeDelayed);
 }
 
 // Any shape: one element per thread step, transposed store.  Used when the tile kernel's
@@ -313,18 +332,15 @@ __global__ __launch_bounds__(kThreads) void quant_transpose_scalar_kernel(
         const int64_t r = j / cols, c = j % cols;
         out_t[c * rows + r] = b;
     }
-    if constexpr (kAmax) publish_and_finalize(L::to_f32_bits(m_run), ws, io, kModeDelayed);
+    if constexpr (kAmax) publish_and_finalize<kThreads>(L::to_f32_bits(m_run), ws, io, kModeDelayed);
 }
 
 // ---------------------------------------------------------------------------------------------
 // Dequantise: out = out_dtype(decode(byte) * (1 / scale)).
 template <int F>
 __device__ __forceinline__ float decode1(uint32_t b) {
-    float v;
-    if constexpr (F == kE4M3) v = __builtin_amdgcn_cvt_f32_fp8((int)b, 0);
-    else v = __builtin_amdgcn_cvt_f32_bf8((int)b, 0);
-    // the hardware conversion returns +0 for the code 0x80; the sign bit is carried over explicitly
-    return __uint_as_float(__float_as_uint(v) | ((b & 0x80u) << 24));
+    if constexpr (F == kE4M3) return __builtin_amdgcn_cvt_f32_fp8((int)b, 0);
+    else return __builtin_amdgcn_cvt_f32_bf8((int)b, 0);
 }
 
 template <int F, int OUT>
@@ -333,7 +349,10 @@ __global__ __launch_bounds__(kThreads) void dequant_kernel(const uint8_t* __rest
     const float inv = 1.0f / *scale_ptr;
     const int64_t stride = (int64_t)gridDim.x * kThreads;
     for (int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x; j < n; j += stride) {
-        const float v = decode1<F>(in[j]) * inv;
+        float v = decode1<F>(in[j]) * inv;
+        // keep the fp32 product a value of its own: folded into a mixed-precision fma (x*y + 0) the
+        // conversion would turn -0 into +0
+        asm volatile("" : "+v"(v));
         if constexpr (OUT == NTFP8_F32) ((float*)out)[j] = v;
         else if constexpr (OUT == NTFP8_F16) ((__half*)out)[j] = __float2half_rn(v);
         else {
@@ -369,14 +388,22 @@ __global__ void update_scale_kernel(const float* amax, const float* old_scale, i
 
 // ---------------------------------------------------------------------------------------------
 // Host-side launchers.
-static int grid_for(int64_t work_items, int per_cu_blocks = 8) {
-    int dev = 0, cus = 256;
-    if (hipGetDevice(&dev) == hipSuccess) {
+static int cu_count() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
         int v = 0;
-        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+        cached[dev] = v;
     }
-    int64_t want = (work_items + kThreads - 1) / kThreads;
-    int64_t cap = (int64_t)cus * per_cu_blocks;
+    return cached[dev];
+}
+
+// blocks for `work_items` thread-steps with `threads` per block, at most `per_cu_blocks` per CU
+static int grid_for(int64_t work_items, int threads = kThreads, int per_cu_blocks = 8) {
+    int64_t want = (work_items + threads - 1) / threads;
+    int64_t cap = (int64_t)cu_count() * per_cu_blocks;
     if (want < 1) want = 1;
     return (int)(want < cap ? want : cap);
 }
@@ -389,16 +416,16 @@ static int launch_flat(int mode, const void* x, int64_t n, bool vec_ok, uint8_t*
     typedef typename ElemOf<S>::type E;
     const int64_t n_vec = vec_ok ? n / kVec : 0;
     // two 16-element groups per lane per trip
-    const int grid = grid_for(n_vec > 0 ? (n_vec + 1) / 2 : n);
+    const int grid = grid_for(n_vec > 0 ? (n_vec + 1) / 2 : n, kFlatThreads, 1);
     const E* xp = static_cast<const E*>(x);
     if (mode == kModeAmaxOnly)
-        hipLaunchKernelGGL((quant_flat_kernel<S, F, kModeAmaxOnly>), dim3(grid), dim3(kThreads), 0, st, xp, n_vec, n, out,
+        hipLaunchKernelGGL((quant_flat_kernel<S, F, kModeAmaxOnly>), dim3(grid), dim3(kFlatThreads), 0, st, xp, n_vec, n, out,
                            scale_ptr, ws, io);
     else if (mode == kModeCastOnly)
-        hipLaunchKernelGGL((quant_flat_kernel<S, F, kModeCastOnly>), dim3(grid), dim3(kThreads), 0, st, xp, n_vec, n, out,
+        hipLaunchKernelGGL((quant_flat_kernel<S, F, kModeCastOnly>), dim3(grid), dim3(kFlatThreads), 0, st, xp, n_vec, n, out,
                            scale_ptr, ws, io);
     else
-        hipLaunchKernelGGL((quant_flat_kernel<S, F, kModeDelayed>), dim3(grid), dim3(kThreads), 0, st, xp, n_vec, n, out,
+        hipLaunchKernelGGL((quant_flat_kernel<S, F, kModeDelayed>), dim3(grid), dim3(kFlatThreads), 0, st, xp, n_vec, n, out,
                            scale_ptr, ws, io);
     return check_launch();
 }
@@ -410,12 +437,13 @@ static int launch_transpose(bool with_amax, const void* x, int64_t rows, int64_t
     const E* xp = static_cast<const E*>(x);
     if (tile_ok) {
         const int64_t tiles = (rows / kTile) * (cols / kTile);
-        if (tiles > 0x7fffffff) return NTFP8_ERR_SIZE;
+        const int64_t cap = (int64_t)cu_count() * (with_amax ? 2 : 8);
+        const int tgrid = (int)(tiles < cap ? tiles : cap);
         if (with_amax)
-            hipLaunchKernelGGL((quant_transpose_kernel<S, F, true>), dim3((int)tiles), dim3(kThreads), 0, st, xp, rows,
+            hipLaunchKernelGGL((quant_transpose_kernel<S, F, true>), dim3(tgrid), dim3(kTileThreads), 0, st, xp, rows,
                                cols, out, out_t, scale_ptr, ws, io);
         else
-            hipLaunchKernelGGL((quant_transpose_kernel<S, F, false>), dim3((int)tiles), dim3(kThreads), 0, st, xp, rows,
+            hipLaunchKernelGGL((quant_transpose_kernel<S, F, false>), dim3(tgrid), dim3(kTileThreads), 0, st, xp, rows,
                                cols, out, out_t, scale_ptr, ws, io);
     } else {
         const int grid = grid_for(rows * cols);
