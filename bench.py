@@ -47,7 +47,7 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=20)
     p.add_argument("--warmup", type=int, default=5)
-    p.add_argument("--workload", choices=["linear", "quant"], default="linear")
+    p.add_argument("--workload", choices=["linear", "quant", "probe"], default="linear")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--kernel-reps", type=int, default=20, help="launches per GEMM shape for the roofline timing")
     return p.parse_args()
@@ -225,6 +225,44 @@ def cpu_baseline_quant():
             "kind": "port", "sample": f"bf16 [4096,4096] delayed-scaling quantise (amax, cast, roll), {2 * n} tensor-steps"}
 
 
+# ------------------------------------------------------------------------------------ counter probe
+def probe(device):
+    """A handful of launches for `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs: one plain copy of
+    known size (the calibration for the counters), the fused quantise kernel on the benchmark tensor,
+    and one GEMM of every kind on the O-projection and gate shapes.  Prints what was launched."""
+    import torch
+
+    from nanotron_amd.fp8 import DTypes, FP8Tensor
+    from nanotron_amd.fp8.kernel import _gemm_nt
+
+    src = torch.empty(128 * 1024 * 1024, dtype=torch.uint8, device=device).fill_(1)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    dst.copy_(src)  # 128 MiB read + 128 MiB written
+    bufs, states = build_quant(device, nbuf=2)
+    for i in range(3):
+        quant_step(bufs, states, i)
+    g = torch.Generator(device="cpu").manual_seed(7)
+    launched = {"copy": {"read_bytes": src.numel(), "write_bytes": src.numel()},
+                "quant_flat_kernel": {"elements": 4096 * 4096, "algorithmic_bytes": 3 * 4096 * 4096}}
+    for name, K, N in (("o", 4096, 4096), ("gate", 4096, 14336)):
+        x = torch.randn(TOKENS, K, generator=g).to(torch.bfloat16).to(device)
+        w = (torch.randn(N, K, generator=g) * 0.02).to(device)
+        gy = (torch.randn(TOKENS, N, generator=g) * 1e-3).to(torch.bfloat16).to(device)
+        xq = FP8Tensor(x, DTypes.FP8E4M3, with_transpose=True)
+        wq = FP8Tensor(w, DTypes.FP8E4M3, with_transpose=True)
+        gq = FP8Tensor(gy, DTypes.FP8E5M2, with_transpose=True)
+        _gemm_nt(xq, wq, torch.bfloat16, None)
+        _gemm_nt(gq, wq.transposed(), torch.bfloat16, None)
+        _gemm_nt(gq.transposed(), xq.transposed(), torch.float32, None)
+        launched[f"gemm_{name}"] = {"M": TOKENS, "N": N, "K": K,
+                                    "algorithmic_bytes_fwd": TOKENS * K + N * K + 2 * TOKENS * N,
+                                    "algorithmic_bytes_dgrad": TOKENS * N + N * K + 2 * TOKENS * K,
+                                    "algorithmic_bytes_wgrad": TOKENS * N + TOKENS * K + 4 * N * K}
+    torch.cuda.synchronize()
+    print(json.dumps({"probe": launched}))
+
+
 # ------------------------------------------------------------------------------------ main
 def main():
     args = parse()
@@ -240,6 +278,9 @@ def main():
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
+    if args.workload == "probe":
+        probe(device)
+        return
     if args.workload == "linear":
         mods, xs, gys = build_linears(device)
         xs = [x.requires_grad_(True) for x in xs]

@@ -69,6 +69,13 @@ __device__ __forceinline__ void mfma_priority(bool high) {
     if (high) __builtin_amdgcn_s_setprio(1);
     else __builtin_amdgcn_s_setprio(0);
 }
+// x of lanes 32..63 <-> y of lanes 0..31 (V_PERMLANE32_SWAP)
+__device__ __forceinline__ void swap_halves(uint32_t& x, uint32_t& y) {
+    typedef unsigned v2u __attribute__((ext_vector_type(2)));
+    const v2u r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
+    x = r.x;
+    y = r.y;
+}
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
@@ -104,6 +111,39 @@ __device__ __forceinline__ void store_wave_tile(const v16f (&acc)[MI][NJ], void*
                                                 int N, int m_base, int n_base, int lane) {
     typedef typename OutT<DT>::type O;
     O* D = static_cast<O*>(Dv);
+    if constexpr (DT != NTFP8_F32) {
+        // 16-bit outputs: a lane's 4 consecutive n are only 8 bytes, and the two 32-lane halves of the
+        // wave hold adjacent groups of 4.  Swapping registers between the halves gives every lane 8
+        // consecutive n (16 bytes), and lanes l / l + 32 together a full 32-byte sector per row, which
+        // is what the memory side writes without read-modify-write traffic.
+        if ((N & 7) == 0) {
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                const int m = m_base + i * 32 + (lane & 31);
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) {
+                        uint32_t w[4];
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const int g = 2 * q + h;
+                            w[2 * h] = (uint32_t)OutT<DT>::cvt(acc[i][j][g * 4 + 0] * alpha) |
+                                       ((uint32_t)OutT<DT>::cvt(acc[i][j][g * 4 + 1] * alpha) << 16);
+                            w[2 * h + 1] = (uint32_t)OutT<DT>::cvt(acc[i][j][g * 4 + 2] * alpha) |
+                                           ((uint32_t)OutT<DT>::cvt(acc[i][j][g * 4 + 3] * alpha) << 16);
+                        }
+                        swap_halves(w[0], w[2]);
+                        swap_halves(w[1], w[3]);
+                        const int n = n_base + j * 32 + (2 * q + (lane >> 5)) * 8;
+                        if (m < M && n < N)
+                            *reinterpret_cast<v4i*>(D + (int64_t)m * N + n) = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+                    }
+                }
+            }
+            return;
+        }
+    }
     const bool vec_ok = (N & 3) == 0;
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
