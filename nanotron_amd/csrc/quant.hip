@@ -158,16 +158,15 @@ __device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, c
         s_last = (t == gridDim.x - 1);
     }
     __syncthreads();
-    if (!s_last || threadIdx.x != 0) return;
+    // The epilogue runs on the first wave of the block that drew the last ticket: every global access
+    // below is one round trip for the whole wave instead of one per history entry.
+    if (!s_last || threadIdx.x >= 64) return;
+    const int lane = threadIdx.x;
     uint32_t bits = 0;
-#pragma unroll
-    for (int i = 0; i < kMaxSlots; ++i) {
-        const uint32_t v = __hip_atomic_load(&ws->slot[i].bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        bits = v > bits ? v : bits;
-    }
+    if (lane < kMaxSlots) bits = __hip_atomic_load(&ws->slot[lane].bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    bits = wave_max_u32(bits);
     if (bits > kInfBits) bits = kNanBits;
     const float a = __uint_as_float(bits);
-    *io.amax_out = a;
     float used;
     if (mode == kModeAmaxOnly) {
         const float old = io.old_scale ? *io.old_scale : 1.0f;
@@ -175,23 +174,28 @@ __device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, c
     } else {
         used = *io.scale_state;
     }
-    if (io.scale_out) *io.scale_out = used;
+    uint32_t hm = bits;
     if (io.hist) {
-        uint32_t hm = bits;
-        for (int i = io.hist_len - 1; i > 0; --i) {
-            const float h = io.hist[i - 1];
-            io.hist[i] = h;
-            uint32_t hb = __float_as_uint(h) & 0x7fffffffu;
+        // hist[i] <- hist[i-1], hist[0] <- a; 64 entries per trip, highest chunk first so that an entry is
+        // read before the chunk below overwrites it
+        for (int base = ((io.hist_len - 1) / 64) * 64; base >= 0; base -= 64) {
+            const int i = base + lane;
+            const bool ok = i < io.hist_len;
+            float h = 0.0f;
+            if (ok) h = (i == 0) ? a : io.hist[i - 1];
+            if (ok) io.hist[i] = h;
+            const uint32_t hb = wave_max_u32(ok ? (__float_as_uint(h) & 0x7fffffffu) : 0u);
             hm = hb > hm ? hb : hm;
         }
-        io.hist[0] = a;
         if (hm > kInfBits) hm = kNanBits;
-        *io.scale_state = update_scale(__uint_as_float(hm), used, io.fmt, io.margin);
     }
-#pragma unroll
-    for (int i = 0; i < kMaxSlots; ++i)
-        __hip_atomic_store(&ws->slot[i].bits, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&ws->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) {
+        *io.amax_out = a;
+        if (io.scale_out) *io.scale_out = used;
+        if (io.hist) *io.scale_state = update_scale(__uint_as_float(hm), used, io.fmt, io.margin);
+        __hip_atomic_store(&ws->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (lane < kMaxSlots) __hip_atomic_store(&ws->slot[lane].bits, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ bool degenerate_scale(float s) {
