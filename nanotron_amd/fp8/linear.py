@@ -36,6 +36,7 @@ class FP8Linear(nn.Linear):
         self.out_dtype = out_dtype
         self.accumulate_grad = accumulate_grad
         self.scaling = None
+        self._weight_ready = None
         if self.weight.device != torch.device("cpu"):
             self.weight = FP8Parameter(self.weight, dtype=DTypes.FP8E4M3)
 
@@ -64,18 +65,40 @@ class FP8Linear(nn.Linear):
                 }
 
     @torch.no_grad()
-    def requantize_weight(self) -> None:
+    def requantize_weight(self, stream: Optional[torch.cuda.Stream] = None) -> None:
         """Refresh the fp8 weight (and its transpose) from the high-precision master copy; with
-        delayed scaling this advances the weight role's amax history by one step."""
+        delayed scaling this advances the weight role's amax history by one step.
+
+        With `stream`, the (HBM-bound) quantisation is queued on that stream behind the work already
+        on the current one, so it overlaps whatever the current stream does next (typically the
+        MFMA-bound GEMMs of other layers); the next forward of this layer waits for it."""
         w = self.weight
         hp = w.as_subclass(torch.Tensor)
         state = self.scaling["weight"] if self.scaling is not None else None
-        w.data = FP8Tensor(hp, dtype=DTypes.FP8E4M3, state=state, with_transpose=True)
+        if stream is None:
+            w.data = FP8Tensor(hp, dtype=DTypes.FP8E4M3, state=state, with_transpose=True)
+            self._weight_ready = None
+            return
+        cur = torch.cuda.current_stream(hp.device)
+        stream.wait_stream(cur)
+        with torch.cuda.stream(stream):
+            q = FP8Tensor(hp, dtype=DTypes.FP8E4M3, state=state, with_transpose=True)
+            ready = torch.cuda.Event()
+            ready.record(stream)
+        # the new tensors were allocated on `stream` and will be read on the current one
+        for t in (q, q.transposed(), q.fp8_meta.amax):
+            t.record_stream(cur)
+        w.data = q
+        self._weight_ready = ready
 
     def forward(self, input: Union[FP8Tensor, torch.Tensor]) -> torch.Tensor:
         # fp8 kernels only when both input and weight are on the GPU (linear.py:53-54)
         if input.device == torch.device("cpu") or self.weight.device == torch.device("cpu"):
             return F.linear(input, self.weight, self.bias)
+
+        if self._weight_ready is not None:  # weight re-quantisation queued on another stream
+            torch.cuda.current_stream(input.device).wait_event(self._weight_ready)
+            self._weight_ready = None
 
         # phony tensor that makes autograd call our backward although the weight's gradient is
         # produced by the fp8 kernels, not by autograd (linear.py:56-60)
