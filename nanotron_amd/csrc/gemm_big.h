@@ -1,0 +1,357 @@
+// Large-tile FP8 GEMM kernel for gfx950; included by gemm.hip after the shared helpers.
+//
+// Block tile (32 MI) x 256 x 128 bytes of K, four waves in a 2 x 2 arrangement, one wave per
+// SIMD.  Each wave owns (16 MI) x 128 outputs as MI x 8 accumulator blocks of V_MFMA_F32_16X16X128_F8F6F4
+// (MI = 8: 256-row block tile, 256 accumulator registers per lane; MI = 4: 128-row block tile).
+//
+// Data movement per K-tile: every wave brings a quarter of the A and B tiles from global memory
+// straight into LDS (16 bytes per lane, XOR-swizzled), reads its MI A fragments from LDS once and
+// keeps them in registers, and streams its 8 B fragments from LDS two MFMA groups ahead of their
+// use.  One MFMA group = the MI MFMAs that share one B fragment.
+//
+// Pipeline, two LDS stages, ONE workgroup barrier per K-tile placed after MFMA group 5:
+//   * before the barrier a wave has read every fragment of the current tile into registers, so after
+//     it the current stage can be refilled with tile kt + 2 (first half of the loads under groups
+//     6-7, second half under groups 0-1 of the next tile);
+//   * the barrier also publishes tile kt + 1 (each wave waits for its own loads first).  Groups 6 and 7
+//     are issued interleaved, two MFMAs per A fragment; the fragment register is dead after them and is
+//     refilled on the spot with the same fragment of tile kt + 1, so one set of A registers suffices.
+// The matrix pipe therefore never waits for LDS or for the barrier's stragglers by more than the
+// skew between waves, and the loads of a tile have more than a full tile of MFMA time to land.
+#pragma once
+
+namespace ntfp8 {
+
+constexpr int kBigN = 256;
+constexpr int kBigWaves = 4, kBigThreads = kBigWaves * 64;
+constexpr int kBigNJ = 8;              // 16-column accumulator blocks per wave: 128 columns
+constexpr int kBigLB = kBigN / 8 / kBigWaves;   // 1 KB wave-level loads of the B tile per wave per stage
+
+// Swizzle for 16-row fragments: the 16 lanes that read chunk c of rows r .. r + 15 hit 16 distinct
+// 16-byte bank groups when the chunk index is XORed with (row mod 8) ^ (bit 3 of row).
+__device__ __forceinline__ int swz16(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+__device__ __forceinline__ int lds_off16(int row, int kc) { return row * kBK + ((kc ^ swz16(row)) << 4); }
+
+template <int FA, int FB>
+__device__ __forceinline__ v4f mfma_16x16x128(v8i b_frag, v8i a_frag, v4f c) {
+    // B fragment first: the 16 x 16 result block is indexed [n][m], so a lane owns 4 consecutive n
+    // (n = 4 (lane / 16) + r) of one output row m = lane % 16.
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b_frag, a_frag, c, FB, FA, 0, 0, 0, 0);
+}
+// rows (groups of 16 lanes) 1 and 3 of x <-> rows 0 and 2 of y (V_PERMLANE16_SWAP)
+__device__ __forceinline__ void swap_rows16(uint32_t& x, uint32_t& y) {
+    typedef unsigned v2u __attribute__((ext_vector_type(2)));
+    const v2u r = __builtin_amdgcn_permlane16_swap(x, y, false, false);
+    x = r.x;
+    y = r.y;
+}
+__device__ __forceinline__ void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
+
+// Epilogue of one wave: MI x NJ accumulator blocks of 16 x 16, block (i, j) at rows m_base + 16 i,
+// columns n_base + 16 j.  Descale, optional fp32 accumulate, one rounding, store.
+template <int DT, bool kAcc, int MI, int NJ>
+__device__ __forceinline__ void store_wave_tile16(const v4f (&acc)[MI][NJ], void* __restrict__ Dv, float alpha, int M,
+                                                  int N, int m_base, int n_base, int lane) {
+    typedef typename OutT<DT>::type O;
+    O* D = static_cast<O*>(Dv);
+    const int mrow = lane & 15, q = lane >> 4;
+    if constexpr (DT != NTFP8_F32) {
+        // 16-bit outputs: a lane's 4 consecutive n are only 8 bytes.  Exchanging registers of two
+        // neighbouring blocks between lane rows gives every lane 8 consecutive n (16 bytes) of one
+        // block, and lane rows r / r + 2 together a full 32-byte sector per output row, which the
+        // memory side writes without read-modify-write traffic.
+        if ((N & 7) == 0) {
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                const int m = m_base + i * 16 + mrow;
+#pragma unroll
+                for (int j = 0; j < NJ; j += 2) {
+                    uint32_t x0 = OutT<DT>::pack2(acc[i][j][0] * alpha, acc[i][j][1] * alpha);
+                    uint32_t x1 = OutT<DT>::pack2(acc[i][j][2] * alpha, acc[i][j][3] * alpha);
+                    uint32_t y0 = OutT<DT>::pack2(acc[i][j + 1][0] * alpha, acc[i][j + 1][1] * alpha);
+                    uint32_t y1 = OutT<DT>::pack2(acc[i][j + 1][2] * alpha, acc[i][j + 1][3] * alpha);
+                    swap_rows16(x0, y0);
+                    swap_rows16(x1, y1);
+                    // lane row q now holds n 8 (q / 2) .. + 7 of block j + (q & 1): x = first four, y = last four
+                    const int n = n_base + (j + (q & 1)) * 16 + (q >> 1) * 8;
+                    if (m < M && n < N)
+                        *reinterpret_cast<v4i*>(D + (int64_t)m * N + n) = (v4i){(int)x0, (int)x1, (int)y0, (int)y1};
+                }
+            }
+            return;
+        }
+    }
+    const bool vec_ok = (N & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+        const int m = m_base + i * 16 + mrow;
+        if (m >= M) continue;
+        // accumulate: all of a row block's old values are requested before the first one is needed
+        v4f old[NJ];
+        if constexpr (kAcc) {
+            if (vec_ok) {
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    const int n = n_base + j * 16 + q * 4;
+                    old[j] = n + 3 < N ? *reinterpret_cast<const v4f*>(static_cast<const float*>(Dv) + (int64_t)m * N + n)
+                                       : (v4f){0.f, 0.f, 0.f, 0.f};
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int n = n_base + j * 16 + q * 4;
+            if (n >= N) continue;
+            O* dp = D + (int64_t)m * N + n;
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[i][j][e] * alpha;
+            if (vec_ok && n + 3 < N) {
+                if constexpr (DT == NTFP8_F32) {
+                    v4f o = {v[0], v[1], v[2], v[3]};
+                    if constexpr (kAcc) o = o + old[j];
+                    *reinterpret_cast<v4f*>(dp) = o;
+                } else {
+                    *reinterpret_cast<uint2*>(dp) = make_uint2(OutT<DT>::pack2(v[0], v[1]), OutT<DT>::pack2(v[2], v[3]));
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (n + e < N) {
+                        if constexpr (DT == NTFP8_F32) {
+                            float o = v[e];
+                            if constexpr (kAcc) o = o + dp[e];
+                            dp[e] = o;
+                        } else {
+                            dp[e] = OutT<DT>::cvt(v[e]);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Launch geometry, computed on the host.  The first `full_blocks` tiles (in grouped order) are computed
+// whole by the MI = 8 kernel.  If the tile count leaves a partial last round over the CUs, the
+// remaining `tail_tiles` tiles are cut into two 128-row halves and computed by a second launch of
+// the MI = 4 kernel with 2 tail_tiles workgroups, so that the last round is half as long.
+struct BigGrid {
+    int tiles_m, tiles_n;   // 256 x 256 tiles
+    int full_blocks;        // tiles computed whole
+    int tail_tiles;         // tiles computed as two halves
+};
+
+// MI = 8 needs the whole register file of a SIMD for one wave (256 accumulators + fragments).  The
+// MI = 4 variant is held to half of it by declaring a launch bound of twice its real workgroup
+// size: given more registers than it needs, the compiler keeps its accumulators in a second
+// register set and copies them back and forth inside the K loop.
+template <int FA, int FB, int DT, bool kAcc, int MI>
+__global__ __launch_bounds__(MI == 8 ? kBigThreads : 2 * kBigThreads)
+void gemm_nt_big_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, void* __restrict__ Dv,
+                        const float* __restrict__ scale_a, const float* __restrict__ scale_b, int M, int N, int K,
+                        BigGrid g) {
+    __shared__ __attribute__((aligned(1024))) uint8_t sA[2][32 * MI * kBK];
+    __shared__ __attribute__((aligned(1024))) uint8_t sB[2][kBigN * kBK];
+
+    // ---- which tile (or half tile) is this workgroup's -------------------------------------------
+    int pid = blockIdx.x;
+    int half = 0;
+    if constexpr (MI == 8) {
+        if (g.full_blocks % kXcds == 0) pid = (pid % kXcds) * (g.full_blocks / kXcds) + pid / kXcds;
+    } else {
+        const int nb = 2 * g.tail_tiles;
+        if (nb % kXcds == 0) pid = (pid % kXcds) * (nb / kXcds) + pid / kXcds;
+        half = pid & 1;
+        pid = g.full_blocks + (pid >> 1);
+    }
+    int pid_m, pid_n;
+    {
+        const int in_group = kGroupM * g.tiles_n;
+        const int group = pid / in_group;
+        const int first_m = group * kGroupM;
+        const int gsz = min(g.tiles_m - first_m, kGroupM);
+        pid_m = first_m + (pid % in_group) % gsz;
+        pid_n = (pid % in_group) / gsz;
+    }
+    const int n0 = pid_n * kBigN;
+    const int m0 = pid_m * 256 + half * 128;
+    if (m0 >= M) return;   // second half of a bottom-edge tile with nothing in it (uniform for the workgroup)
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    // the wave index as a scalar: LDS destinations of the loads (M0) and every other per-wave offset then
+    // live in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(A, (uint32_t)((int64_t)M * K));
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(B, (uint32_t)((int64_t)N * K));
+    const int KT = (K + kBK - 1) / kBK;   // >= 2 (host)
+    // A wave-level load fills 8 tile rows (1 KB of LDS, lane i at byte 16 i); the lane landing on
+    // chunk position p of row r fetches global chunk p ^ swz16(r).  For the rows a lane serves
+    // (8 (wave + 4 i) + lane / 8) that is the same chunk for every i.
+    const int ld_kc = ((lane & 7) ^ (lane >> 3) ^ (wave & 1)) << 4;
+    // chunks of the last K-tile at k >= K must read as zero, not as the start of the next row
+    const bool tail_dead = (KT - 1) * kBK + ld_kc >= K;
+    const float alpha = (1.0f / *scale_a) * (1.0f / *scale_b);
+
+    {
+        constexpr int LA = MI * 2 * 16 / 8 / kBigWaves;  // wave-level loads of the A tile per wave per stage
+        constexpr int LB = kBigLB;
+        constexpr int NL = LA + LB;                      // loads per wave per K-tile
+        static_assert(NL % 4 == 0, "the loads are queued in four equal portions");
+        const int wm = (wave >> 1) * (MI * 16), wn = (wave & 1) * 128;
+
+        uint32_t a_off[LA], b_off[LB];
+#pragma unroll
+        for (int i = 0; i < LA; ++i)   // rows >= M fall past the descriptor: zeros
+            a_off[i] = (uint32_t)(m0 + (wave + kBigWaves * i) * 8 + (lane >> 3)) * (uint32_t)K + ld_kc;
+#pragma unroll
+        for (int i = 0; i < LB; ++i)
+            b_off[i] = (uint32_t)(n0 + (wave + kBigWaves * i) * 8 + (lane >> 3)) * (uint32_t)K + ld_kc;
+
+        v4f acc[MI][kBigNJ];
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < kBigNJ; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+        // load number `l` (0 .. NL-1, A loads first) of K-tile `ktile` into stage `s`
+        auto issue = [&](int s, int ktile, int l) {
+            if (l < LA)
+                lds_load16(ra, (lds_ptr)(uintptr_t)&sA[s][(wave + kBigWaves * l) * 1024], a_off[l], ktile * kBK);
+            else
+                lds_load16(rb, (lds_ptr)(uintptr_t)&sB[s][(wave + kBigWaves * (l - LA)) * 1024], b_off[l - LA], ktile * kBK);
+        };
+        // Called once, before the first load of the last K-tile is queued (no other tile is loaded after it):
+        // lanes whose chunk lies at k >= K get an offset past the descriptor and so read zeros.
+        auto poison_tail = [&]() {
+            if (tail_dead) {
+#pragma unroll
+                for (int i = 0; i < LA; ++i) a_off[i] = 0xfffffff0u;
+#pragma unroll
+                for (int i = 0; i < LB; ++i) b_off[i] = 0xfffffff0u;
+            }
+        };
+
+        // fragment reads: lane -> row (lane % 16) of a 16-row block, two 16-byte chunks 2 (lane / 16) + {0, 1};
+        // block i of the wave is 16 i rows = 2048 i bytes further on (the swizzle only looks at row bits 0-3)
+        const int frow = lane & 15;
+        const int fk = (lane >> 4) * 2;
+        const int a_rd0 = lds_off16(wm + frow, fk), a_rd1 = lds_off16(wm + frow, fk + 1);
+        const int b_rd0 = lds_off16(wn + frow, fk), b_rd1 = lds_off16(wn + frow, fk + 1);
+        // half h (0 / 1) of a fragment = one 128-bit LDS read
+        auto rd_a = [&](int s, int i, int h) -> v4i {
+            return *reinterpret_cast<const v4i*>(&sA[s][(h ? a_rd1 : a_rd0) + i * 2048]);
+        };
+        auto rd_b = [&](int s, int j, int h) -> v4i {
+            return *reinterpret_cast<const v4i*>(&sB[s][(h ? b_rd1 : b_rd0) + j * 2048]);
+        };
+        auto frag = [](const v4i (&x)[2]) -> v8i { return (v8i){x[0].x, x[0].y, x[0].z, x[0].w, x[1].x, x[1].y, x[1].z, x[1].w}; };
+
+        v4i fa[MI][2], fb[4][2];
+
+        // A K-tile kt lives in LDS stage kt & 1 and is computed in two parts:
+        //   front(kt): MFMA groups 0-5.  Entered with fa[] = the tile's A fragments and fb[0], fb[1] = its first
+        //              two B fragments; streams B fragments 2..7; queues the loads of tile kt + 1 that are not
+        //              yet queued; ends with the barrier that publishes tile kt + 1 and releases stage kt & 1.
+        //   back(kt):  MFMA groups 6-7, interleaved per A fragment; refills fa[] / fb[0], fb[1] from tile kt + 1
+        //              and queues the first kBackLoads loads of tile kt + 2 into the released stage.
+        // The K loop runs back(kt); front(kt + 1), so that its back edge sits right behind the barrier, where no
+        // LDS read is outstanding.
+        //
+        // An MFMA occupies the matrix pipe for 32 cycles and the wave issues in order, so whatever stands between
+        // two MFMAs must issue within that time or the pipe idles.  The code below therefore puts at most one
+        // memory instruction (two LDS reads at most) behind each MFMA, and a scheduling fence behind each such
+        // pair keeps the compiler from regrouping them.
+        constexpr int kBackLoads = NL / 2;
+        constexpr int kFrontLoads = NL - kBackLoads;   // half under group 0, half under group 1
+        auto front = [&](auto loads_tag, auto barrier_tag, int kt) {
+            constexpr bool loads = decltype(loads_tag)::value, barrier = decltype(barrier_tag)::value;
+            const int s = kt & 1;
+            sched_fence();
+#pragma unroll
+            for (int j = 0; j < 6; ++j) {
+                int l = kBackLoads + j * (kFrontLoads / 2);           // next load of tile kt + 1 to queue
+                const int lend = (loads && j < 2) ? l + kFrontLoads / 2 : l;
+#pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    acc[i][j] = mfma_16x16x128<FA, FB>(frag(fb[j & 3]), frag(fa[i]), acc[i][j]);
+                    if (i == 0) fb[(j + 2) & 3][0] = rd_b(s, j + 2, 0);
+                    else if (i == 2) fb[(j + 2) & 3][1] = rd_b(s, j + 2, 1);
+                    else if (l < lend) issue(s ^ 1, kt + 1, l++);
+                    if (i == MI - 1) {   // whatever did not get a slot of its own
+                        for (; l < lend; ++l) issue(s ^ 1, kt + 1, l);
+                    }
+                    sched_fence();
+                }
+            }
+            if constexpr (barrier) {
+                // Every fragment of tile kt is in registers (or in flight): after the barrier stage s may be
+                // overwritten, and tile kt + 1 is complete in stage s ^ 1.
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                wg_barrier();
+            }
+        };
+        auto back = [&](auto loads_tag, auto prefetch_tag, int kt) {
+            constexpr bool loads = decltype(loads_tag)::value, prefetch = decltype(prefetch_tag)::value;
+            const int s = kt & 1;
+            if (loads && kt + 3 == KT) poison_tail();   // the loads queued below are the first of the last tile
+            sched_fence();
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                // fa[i] is dead after its two MFMAs; it is refilled with the fragment of the next tile one step later
+                acc[i][6] = mfma_16x16x128<FA, FB>(frag(fb[2]), frag(fa[i]), acc[i][6]);
+                if (prefetch && i > 0) {
+                    fa[i - 1][0] = rd_a(s ^ 1, i - 1, 0);
+                    fa[i - 1][1] = rd_a(s ^ 1, i - 1, 1);
+                }
+                sched_fence();
+                acc[i][7] = mfma_16x16x128<FA, FB>(frag(fb[3]), frag(fa[i]), acc[i][7]);
+                if constexpr (loads) {   // loads [i kBackLoads / MI, (i + 1) kBackLoads / MI) ride on this step
+#pragma unroll
+                    for (int l = i * kBackLoads / MI; l < (i + 1) * kBackLoads / MI; ++l) issue(s, kt + 2, l);
+                }
+                if (prefetch && i < 4) fb[i >> 1][i & 1] = rd_b(s ^ 1, i >> 1, i & 1);
+                sched_fence();
+            }
+            if constexpr (prefetch) {
+                fa[MI - 1][0] = rd_a(s ^ 1, MI - 1, 0);
+                fa[MI - 1][1] = rd_a(s ^ 1, MI - 1, 1);
+            }
+            sched_fence();
+        };
+        using Yes = std::true_type;
+        using No = std::false_type;
+
+        // prologue: tile 0 completely, the first kBackLoads loads of tile 1
+#pragma unroll
+        for (int l = 0; l < NL; ++l) issue(0, 0, l);
+        if (KT == 2) poison_tail();
+#pragma unroll
+        for (int l = 0; l < kBackLoads; ++l) issue(1, 1, l);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBackLoads) : "memory");
+        wg_barrier();
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            fa[i][0] = rd_a(0, i, 0);
+            fa[i][1] = rd_a(0, i, 1);
+        }
+#pragma unroll
+        for (int h = 0; h < 4; ++h) fb[h >> 1][h & 1] = rd_b(0, h >> 1, h & 1);
+
+        front(Yes{}, Yes{}, 0);
+        int kt = 0;
+        for (; kt < KT - 2; ++kt) {
+            back(Yes{}, Yes{}, kt);
+            front(Yes{}, Yes{}, kt + 1);
+        }
+        back(No{}, Yes{}, kt);        // kt = KT - 2: nothing left to load
+        front(No{}, No{}, kt + 1);
+        back(No{}, No{}, kt + 1);
+
+        store_wave_tile16<DT, kAcc, MI, kBigNJ>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
+    }
+}
+
+}  // namespace ntfp8

@@ -1,0 +1,197 @@
+// Helpers shared by the FP8 GEMM kernels: vector types, output conversion, LDS/buffer primitives,
+// tile ordering and the epilogue for 32 x 32 accumulator blocks.
+#pragma once
+#include <type_traits>
+
+#include "common.h"
+
+namespace ntfp8 {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+constexpr int kBK = 128;     // bytes of K per LDS stage
+constexpr int kGroupM = 8;   // tile-order grouping for L2 reuse
+constexpr int kXcds = 8;     // workgroups are dealt round-robin to the 8 XCDs, each with its own L2
+
+// 16-byte chunk `kc` (0..7) of tile row `row`, swizzled so that the 16 lanes of a 128-bit LDS access
+// that read the same chunk of 16 consecutive rows touch 16 distinct 16-byte bank groups.
+__device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
+__device__ __forceinline__ int lds_off(int row, int kc) { return row * kBK + ((kc ^ swz(row)) << 4); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float v) {
+    const uint32_t u = __float_as_uint(v);
+    if ((u & 0x7fffffffu) > kInfBits) return (uint16_t)((u >> 16) | 0x40u);
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+
+// Output element types.  cvt() rounds one value, pack2() two values into one 32-bit word (first value
+// in the low half) with the packed hardware conversions (V_CVT_PK_BF16_F32 / V_CVT_PK_F16_F32, both
+// round-to-nearest-even).
+template <int D>
+struct OutT;
+template <>
+struct OutT<NTFP8_F32> {
+    typedef float type;
+    __device__ static __forceinline__ float cvt(float v) { return v; }
+};
+template <>
+struct OutT<NTFP8_BF16> {
+    typedef uint16_t type;
+    __device__ static __forceinline__ uint16_t cvt(float v) { return f32_to_bf16_rne(v); }
+    __device__ static __forceinline__ uint32_t pack2(float a, float b) {
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector((v2f){a, b}, v2bf));
+    }
+};
+template <>
+struct OutT<NTFP8_F16> {
+    typedef uint16_t type;
+    __device__ static __forceinline__ uint16_t cvt(float v) {
+        asm volatile("" : "+v"(v));  // no folding of the descale multiply into a mixed-precision fma (-0 would become +0)
+        return __half_as_ushort(__float2half_rn(v));
+    }
+    __device__ static __forceinline__ uint32_t pack2(float a, float b) {
+        asm volatile("" : "+v"(a), "+v"(b));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector((v2f){a, b}, v2h));
+    }
+};
+
+// Device-only builtins live in __device__ helpers: written directly inside a __global__ template they
+// are non-dependent expressions that the host pass cannot resolve.
+__device__ __forceinline__ void wg_barrier() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+}
+__device__ __forceinline__ void mfma_priority(bool high) {
+    if (high) __builtin_amdgcn_s_setprio(1);
+    else __builtin_amdgcn_s_setprio(0);
+}
+// x of lanes 32..63 <-> y of lanes 0..31 (V_PERMLANE32_SWAP)
+__device__ __forceinline__ void swap_halves(uint32_t& x, uint32_t& y) {
+    typedef unsigned v2u __attribute__((ext_vector_type(2)));
+    const v2u r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
+    x = r.x;
+    y = r.y;
+}
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+// 16 bytes per lane from global memory straight into LDS: lane i lands at dst + 16 * i.  Offsets past
+// the descriptor's size read as zero.
+__device__ __forceinline__ void lds_load16(__amdgpu_buffer_rsrc_t r, lds_ptr dst, uint32_t voff, int soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, dst, 16, voff, soff, 0, 0);
+}
+template <int FA, int FB>
+__device__ __forceinline__ v16f mfma_32x32x64(v8i b_frag, v8i a_frag, v16f c) {
+    // The B-matrix fragment is the first source, so the 32x32 result block is indexed [n][m]: each
+    // lane then owns 4 consecutive n of one output row m.
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b_frag, a_frag, c, FB, FA, 0, 0, 0, 0);
+}
+
+// tile order: XCD-contiguous, then kGroupM row-tiles swept before moving along N
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int& pid_m, int& pid_n) {
+    int pid = blockIdx.x;
+    const int nwg = gridDim.x;
+    if (nwg % kXcds == 0) pid = (pid % kXcds) * (nwg / kXcds) + pid / kXcds;
+    const int in_group = kGroupM * tiles_n;
+    const int group = pid / in_group;
+    const int first_m = group * kGroupM;
+    const int gsz = min(tiles_m - first_m, kGroupM);
+    pid_m = first_m + (pid % in_group) % gsz;
+    pid_n = (pid % in_group) / gsz;
+}
+
+// Epilogue of one wave: MI x NJ accumulator blocks of 32 x 32, block (i, j) at rows m_base + 32 i,
+// columns n_base + 32 j.  Descale, optional fp32 accumulate, one rounding, store.
+template <int DT, bool kAcc, int MI, int NJ>
+__device__ __forceinline__ void store_wave_tile(const v16f (&acc)[MI][NJ], void* __restrict__ Dv, float alpha, int M,
+                                                int N, int m_base, int n_base, int lane) {
+    typedef typename OutT<DT>::type O;
+    O* D = static_cast<O*>(Dv);
+    if constexpr (DT != NTFP8_F32) {
+        // 16-bit outputs: a lane's 4 consecutive n are only 8 bytes, and the two 32-lane halves of the
+        // wave hold adjacent groups of 4.  Swapping registers between the halves gives every lane 8
+        // consecutive n (16 bytes), and lanes l / l + 32 together a full 32-byte sector per row, which
+        // is what the memory side writes without read-modify-write traffic.
+        if ((N & 7) == 0) {
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                const int m = m_base + i * 32 + (lane & 31);
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) {
+                        uint32_t w[4];
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const int g = 2 * q + h;
+                            w[2 * h] = OutT<DT>::pack2(acc[i][j][g * 4 + 0] * alpha, acc[i][j][g * 4 + 1] * alpha);
+                            w[2 * h + 1] = OutT<DT>::pack2(acc[i][j][g * 4 + 2] * alpha, acc[i][j][g * 4 + 3] * alpha);
+                        }
+                        swap_halves(w[0], w[2]);
+                        swap_halves(w[1], w[3]);
+                        const int n = n_base + j * 32 + (2 * q + (lane >> 5)) * 8;
+                        if (m < M && n < N)
+                            *reinterpret_cast<v4i*>(D + (int64_t)m * N + n) = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+                    }
+                }
+            }
+            return;
+        }
+    }
+    const bool vec_ok = (N & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+        const int m = m_base + i * 32 + (lane & 31);
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n_base + j * 32 + g * 8 + (lane >> 5) * 4;
+                if (n >= N) continue;
+                O* dp = D + (int64_t)m * N + n;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e] * alpha;
+                if (vec_ok && n + 3 < N) {
+                    if constexpr (DT == NTFP8_F32) {
+                        v4f o = {v[0], v[1], v[2], v[3]};
+                        if constexpr (kAcc) {
+                            const v4f old = *reinterpret_cast<const v4f*>(dp);
+                            o = o + old;
+                        }
+                        *reinterpret_cast<v4f*>(dp) = o;
+                    } else {
+                        const uint32_t lo = OutT<DT>::pack2(v[0], v[1]);
+                        const uint32_t hi = OutT<DT>::pack2(v[2], v[3]);
+                        *reinterpret_cast<uint2*>(dp) = make_uint2(lo, hi);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (n + e < N) {
+                            if constexpr (DT == NTFP8_F32) {
+                                float o = v[e];
+                                if constexpr (kAcc) o = o + dp[e];
+                                dp[e] = o;
+                            } else {
+                                dp[e] = OutT<DT>::cvt(v[e]);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+}  // namespace ntfp8

@@ -392,18 +392,6 @@ __global__ void update_scale_kernel(const float* amax, const float* old_scale, i
 
 // ---------------------------------------------------------------------------------------------
 // Host-side launchers.
-static int cu_count() {
-    static int cached[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int v = 0;
-        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
-        cached[dev] = v;
-    }
-    return cached[dev];
-}
-
 // blocks for `work_items` thread-steps with `threads` per block, at most `per_cu_blocks` per CU
 static int grid_for(int64_t work_items, int threads = kThreads, int per_cu_blocks = 8) {
     int64_t want = (work_items + threads - 1) / threads;

@@ -26,3 +26,15 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(autouse=True)
+def _seed_torch():
+    # the tests mirrored from the reference draw unseeded randn inputs against an absolute tolerance;
+    # a fixed seed per test makes their outcome reproducible
+    import torch
+
+    torch.manual_seed(1234)
+    if torch.cuda.is_available():
+        torch.cuda.manual_seed_all(1234)
+    yield

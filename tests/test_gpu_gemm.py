@@ -67,6 +67,33 @@ def test_integer_operands_bit_exact(fa, fb, mnk):
     assert torch.equal(gpu_gemm_nt(A2, B2).cpu(), want * 0.5)
 
 
+@pytest.mark.parametrize("mnk,fa,fb", [
+    ((4096, 4096, 272), O.E4M3, O.E4M3),    # 256 whole 256x256 tiles (one per CU), K tail of 16
+    ((4096, 6144, 256), O.E5M2, O.E4M3),    # 384 tiles: one whole round + 128 tiles as 128-row halves; two K-tiles
+    ((4000, 4136, 400), O.E4M3, O.E5M2),    # 272 tiles with ragged bottom / right edges, odd K-tile count
+    ((2304, 2048, 1024), O.E4M3, O.E4M3),   # 72 tiles: every tile computed as halves
+])
+def test_large_grid_bit_exact(mnk, fa, fb):
+    """Shapes with enough tiles for the whole-tile kernel (the small shapes above only reach the
+    half-tile one); small integers keep every partial sum exact, so any order must give these bits."""
+    M, N, K = mnk
+    g = torch.Generator().manual_seed(M + 3 * N + 5 * K)
+    a = torch.randint(-4, 5, (M, K), generator=g).float()
+    b = torch.randint(-4, 5, (N, K), generator=g).float()
+    one = torch.tensor(1.0)
+    aq, bq = O.cast_to_fp8(a, one, fa), O.cast_to_fp8(b, one, fb)
+    want = (a @ b.t())  # |sum| <= 16 K < 2^24: exact in fp32 in any order
+    A, B = from_bytes(aq, 1.0, fa), from_bytes(bq, 1.0, fb)
+    assert torch.equal(gpu_gemm_nt(A, B).cpu(), want)
+    for od in (torch.bfloat16, torch.float16):
+        assert torch.equal(gpu_gemm_nt(A, B, od).cpu(), want.to(od))
+    acc = torch.randint(-100, 100, (M, N), generator=g).float()
+    accg = acc.cuda()
+    assert torch.equal(gpu_gemm_nt(A, B, torch.float32, accg).cpu(), want + acc)
+    A2, B2 = from_bytes(aq, 0.25, fa), from_bytes(bq, 8.0, fb)
+    assert torch.equal(gpu_gemm_nt(A2, B2, torch.bfloat16).cpu(), (want * 0.5).to(torch.bfloat16))
+
+
 def test_every_fp8_code_decodes_like_the_oracle():
     # A = one row per code (one-hot in K), B = identity-like selectors: D[i, j] = decode(code i) * [i == j]
     for fmt in FMTS:
