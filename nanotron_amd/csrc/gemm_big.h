@@ -45,6 +45,10 @@ __device__ __forceinline__ void swap_rows16(uint32_t& x, uint32_t& y) {
     x = r.x;
     y = r.y;
 }
+// 16 bytes per lane from global memory into registers; offsets past the descriptor read as zero
+__device__ __forceinline__ v4i reg_load16(__amdgpu_buffer_rsrc_t r, uint32_t voff, int soff) {
+    return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
 __device__ __forceinline__ void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
 
 // Epilogue of one wave: MI x NJ accumulator blocks of 16 x 16, block (i, j) at rows m_base + 16 i,
@@ -324,6 +328,94 @@ void gemm_nt_big_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict
         using Yes = std::true_type;
         using No = std::false_type;
 
+        if constexpr (MI == 8) {
+            // ---- whole tiles: loads staged through registers ------------------------------------------
+            // g[] always holds one K-tile in flight.  front(f) runs between the barriers B(f-1) and B(f); there
+            // g[l] (tile f + 1, requested one K-tile earlier) is written to the stage released by B(f-1) and
+            // at once re-requested for tile f + 2.  Every load so has a full K-tile of MFMA time to arrive
+            // whatever its position, and the requests are spread evenly over the K-tile; with direct-to-LDS
+            // loads (which can only be issued once their stage is free) operands that come from HBM rather
+            // than from the memory-side cache stalled the barrier.
+            v4i g[NL];
+            const int wr_lane = wave * 1024 + lane * 16;   // a wave-level load covers 1 KB of a stage: 16 bytes per lane
+            auto request = [&](int ktile, int l) {
+                g[l] = l < LA ? reg_load16(ra, a_off[l], ktile * kBK) : reg_load16(rb, b_off[l - LA], ktile * kBK);
+            };
+            auto deposit = [&](int s, int l) {
+                if (l < LA) *reinterpret_cast<v4i*>(&sA[s][wr_lane + l * (kBigWaves * 1024)]) = g[l];
+                else *reinterpret_cast<v4i*>(&sB[s][wr_lane + (l - LA) * (kBigWaves * 1024)]) = g[l];
+            };
+            // MFMA groups 0-5 of tile f.  W: deposit tile f + 1; L: request tile f + 2; B: barrier that publishes
+            // tile f + 1.  A group has 8 MFMA slots: two carry the LDS reads of B fragment j + 2, the other six
+            // take deposit / request pairs (three pairs in groups 0-4, the sixteenth pair in group 5).
+            auto front_st = [&](auto w_tag, auto l_tag, auto b_tag, int f) {
+                constexpr bool W = decltype(w_tag)::value, L = decltype(l_tag)::value, B = decltype(b_tag)::value;
+                const int s = f & 1;
+                sched_fence();
+                int l = 0;
+#pragma unroll
+                for (int j = 0; j < 6; ++j) {
+#pragma unroll
+                    for (int i = 0; i < MI; ++i) {
+                        acc[i][j] = mfma_16x16x128<FA, FB>(frag(fb[j & 3]), frag(fa[i]), acc[i][j]);
+                        if (i == 0) fb[(j + 2) & 3][0] = rd_b(s, j + 2, 0);
+                        else if (i == 2) fb[(j + 2) & 3][1] = rd_b(s, j + 2, 1);
+                        else if (l < NL) {
+                            const bool second = i == 3 || i == 5 || i == 7;   // slots 1,3 / 4,5 / 6,7 form the pairs
+                            if (!second) { if (W) deposit(s ^ 1, l); }
+                            else { if (L) request(f + 2, l); ++l; }
+                        }
+                        sched_fence();
+                    }
+                }
+                if constexpr (B) {
+                    // Every fragment of tile f is in registers (or in flight) and this wave's part of tile f + 1 is
+                    // written: after the barrier stage s may be overwritten and tile f + 1 is complete in s ^ 1.
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    wg_barrier();
+                }
+            };
+            // prologue: tiles 0 and 1 straight into LDS
+#pragma unroll
+            for (int l = 0; l < NL; ++l) issue(0, 0, l);
+            if (KT == 2) poison_tail();
+#pragma unroll
+            for (int l = 0; l < NL; ++l) issue(1, 1, l);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            wg_barrier();
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+                fa[i][0] = rd_a(0, i, 0);
+                fa[i][1] = rd_a(0, i, 1);
+            }
+#pragma unroll
+            for (int h = 0; h < 4; ++h) fb[h >> 1][h & 1] = rd_b(0, h >> 1, h & 1);
+
+            // (poison_tail() runs right before the front that requests the last tile, KT - 1 = f + 2)
+            if (KT == 3) poison_tail();
+            if (KT > 2) front_st(No{}, Yes{}, No{}, 0);   // tile 1 is in place already; nothing to publish or release
+            else front_st(No{}, No{}, No{}, 0);
+            int f = 1;
+            for (; f + 3 < KT; ++f) {
+                back(No{}, Yes{}, f - 1);
+                front_st(Yes{}, Yes{}, Yes{}, f);
+            }
+            if (f + 2 < KT) {   // f = KT - 3 >= 1
+                poison_tail();
+                back(No{}, Yes{}, f - 1);
+                front_st(Yes{}, Yes{}, Yes{}, f);
+                ++f;
+            }
+            if (f + 1 < KT) {   // f = KT - 2 >= 1: the last tile is deposited, nothing left to request
+                back(No{}, Yes{}, f - 1);
+                front_st(Yes{}, No{}, Yes{}, f);
+                ++f;
+            }
+            back(No{}, Yes{}, f - 1);   // f = KT - 1
+            front_st(No{}, No{}, No{}, f);
+            back(No{}, No{}, f);
+        } else {
+        // ---- half tiles: loads go straight into LDS (the register budget has no room for staging) --------
         // prologue: tile 0 completely, the first kBackLoads loads of tile 1
 #pragma unroll
         for (int l = 0; l < NL; ++l) issue(0, 0, l);
@@ -349,6 +441,7 @@ void gemm_nt_big_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict
         back(No{}, Yes{}, kt);        // kt = KT - 2: nothing left to load
         front(No{}, No{}, kt + 1);
         back(No{}, No{}, kt + 1);
+        }
 
         store_wave_tile16<DT, kAcc, MI, kBigNJ>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
     }
