@@ -76,16 +76,16 @@ def event_time_ms(fn, reps, warm=3):
 def build_linears(device):
     import torch
 
-    from nanotron_amd.fp8 import FP8Linear
+    from nanotron_amd.fp8 import DTypes, FP8Linear, FP8Parameter
 
     g = torch.Generator(device="cpu").manual_seed(1234 + 500)
     mods, xs, gys = [], [], []
     for name, K, N in LINEARS:
         lin = FP8Linear(K, N, bias=False, device=device, out_dtype=torch.bfloat16, delayed_scaling=True,
                         amax_history_len=16, margin=0)
-        w = (torch.randn(N, K, generator=g, dtype=torch.float32) * 0.02)
-        with torch.no_grad():
-            lin.weight.as_subclass(torch.Tensor).copy_(w.to(device))
+        # bf16 master weights ~N(0, 0.02), re-quantised (delayed scaling) every step
+        w = (torch.randn(N, K, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+        lin.weight = FP8Parameter(w.to(device), DTypes.FP8E4M3)
         mods.append(lin)
         xs.append((torch.randn(TOKENS, K, generator=g, dtype=torch.float32)).to(torch.bfloat16).to(device))
         gys.append((torch.randn(TOKENS, N, generator=g, dtype=torch.float32) * 1e-3).to(torch.bfloat16).to(device))
@@ -360,7 +360,7 @@ def main():
         achieved = gf / (gms * 1e-3) / 1e12
         out.update({
             "metric": "FP8Linear fwd+bwd TFLOP/s", "value": round(value, 2), "unit": "TFLOP/s", "dtype": "fp8",
-            "config": {"workload": "llama3-8b decoder-block linears fwd+bwd, 4096 tokens, delayed scaling hist 16",
+            "config": {"workload": "llama3-8b decoder-block linears fwd+bwd, 4096 tokens, bf16 activations and weights, delayed scaling hist 16",
                        "weight_requantisation": "second stream" if args.weight_stream else "compute stream",
                        "tokens": TOKENS, "linears": [f"{n}:{k}->{o}" for n, k, o in LINEARS],
                        "flops_per_step": flops_step, "pct_fp8_peak": round(100 * value / PEAK_FP8_TFLOPS, 2)},

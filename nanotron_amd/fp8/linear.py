@@ -27,7 +27,8 @@ class FP8Linear(nn.Linear):
     reference's behaviour: `out_dtype` (None = fp32 output, kernel.py:24,28), `delayed_scaling`
     (False = scale every tensor from its own amax), `amax_history_len`, `margin`,
     `accumulate_grad` (False = `weight.grad` is overwritten each backward, linear.py:110; True =
-    the wgrad GEMM adds into the existing fp32 `weight.grad` in its epilogue)."""
+    the wgrad GEMM adds into the existing fp32 gradient in its epilogue).  With a bf16 / fp16
+    master weight the fp32 weight gradient is stored as `weight.main_grad` instead of `.grad`."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, device: Optional[torch.device] = None,
                  *, out_dtype: Optional[torch.dtype] = None, delayed_scaling: bool = False,
@@ -160,13 +161,19 @@ class _FP8Matmul(torch.autograd.Function):
                 grad_input = grad_input.reshape(ctx.in_shape)
         if weight.requires_grad:
             # dW[N,K] = dY[M,N]^T . X[M,K]
+            # The gradient is fp32 (kernel.py:24).  An fp32 parameter takes it as `.grad` (side effect, as
+            # linear.py:110); a 16-bit parameter cannot hold an fp32 `.grad`, so there it is kept beside the
+            # parameter as `.main_grad`, the fp32 master-gradient buffer an optimizer reads.
+            slot = "grad" if weight.dtype == torch.float32 else "main_grad"
             acc = None
-            if module.accumulate_grad and weight.grad is not None and weight.grad.dtype == torch.float32:
-                acc = weight.grad
+            if module.accumulate_grad:
+                prev = getattr(weight, slot, None)
+                if prev is not None and prev.dtype == torch.float32:
+                    acc = prev
             grad_weight = fp8_matmul_kernel(
                 mat_a=input, transpose_a=False, mat_b=grad_output, transpose_b=True, use_split_accumulator=True,
                 accumulate_into=acc,
             )
-            weight.grad = grad_weight  # side effect, as linear.py:110
+            setattr(weight, slot, grad_weight)
 
         return grad_input, None, None, None

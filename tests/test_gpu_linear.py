@@ -167,6 +167,31 @@ def test_accumulate_grad_into_fp32_master_buffer():
         assert O.rel_l2(lin.weight.grad.cpu(), total) <= REL_L2
 
 
+def test_bf16_master_weight_keeps_fp32_gradient_as_main_grad():
+    # bf16 parameters cannot carry an fp32 `.grad`: the fp32 wgrad result goes to `.main_grad`
+    from nanotron_amd.fp8 import DTypes, FP8Linear, FP8Parameter
+
+    M, K, N = 320, 256, 384
+    w = O.normal_tensor(41, (N, K), 0.02, torch.bfloat16)
+    for accumulate in (False, True):
+        lin = FP8Linear(K, N, bias=False, device="cuda", out_dtype=torch.bfloat16, accumulate_grad=accumulate)
+        lin.weight = FP8Parameter(w.cuda(), DTypes.FP8E4M3)
+        assert lin.weight.dtype == torch.bfloat16
+        total = torch.zeros(N, K)
+        for step in range(2):
+            x = O.normal_tensor(50 + step, (M, K), 1.0, torch.bfloat16)
+            gy = O.normal_tensor(60 + step, (M, N), 1e-3, torch.bfloat16)
+            xg = x.cuda().requires_grad_(True)
+            lin.requantize_weight()
+            lin(xg).backward(gy.cuda())
+            *_, dx_ref, dw_ref = _oracle_step(x, w, gy)
+            total = total + dw_ref if accumulate else dw_ref
+            assert lin.weight.grad is None
+            assert lin.weight.main_grad.dtype == torch.float32
+            assert O.rel_l2(lin.weight.main_grad.cpu(), total) <= REL_L2
+            assert O.rel_l2(xg.grad.float().cpu(), dx_ref) <= 4e-3  # bf16 input gradient
+
+
 def test_delayed_scaling_ten_steps_llama_like_block_reduced():
     """Benchmark config 5 in miniature (same structure: 5 linears, fwd+bwd, 10 steps, history 16,
     weights perturbed every step), every amax / scale / history compared bit-exact per step."""
