@@ -372,6 +372,9 @@ void gemm_nt_big_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict
                     // Every fragment of tile f is in registers (or in flight) and this wave's part of tile f + 1 is
                     // written: after the barrier stage s may be overwritten and tile f + 1 is complete in s ^ 1.
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    // the first front publishes tile 1, which the prologue sent straight to LDS: its loads are
+                    // older than the NL requests of tile 2 queued above
+                    if constexpr (!W) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(L ? NL : 0) : "memory");
                     wg_barrier();
                 }
             };
@@ -381,7 +384,7 @@ void gemm_nt_big_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict
             if (KT == 2) poison_tail();
 #pragma unroll
             for (int l = 0; l < NL; ++l) issue(1, 1, l);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");   // tile 0 has landed, tile 1 may still be in flight
             wg_barrier();
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
@@ -393,8 +396,8 @@ void gemm_nt_big_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict
 
             // (poison_tail() runs right before the front that requests the last tile, KT - 1 = f + 2)
             if (KT == 3) poison_tail();
-            if (KT > 2) front_st(No{}, Yes{}, No{}, 0);   // tile 1 is in place already; nothing to publish or release
-            else front_st(No{}, No{}, No{}, 0);
+            if (KT > 2) front_st(No{}, Yes{}, Yes{}, 0);   // nothing to deposit: tile 1 is on its way to LDS already
+            else front_st(No{}, No{}, Yes{}, 0);
             int f = 1;
             for (; f + 3 < KT; ++f) {
                 back(No{}, Yes{}, f - 1);
