@@ -20,11 +20,12 @@ constexpr uint32_t kNanBits = 0x7fc00000u;
 // MI355X), atomics on different lines proceed in parallel.
 constexpr int kMaxSlots = 8;
 struct Workspace {
-    uint32_t ticket;  // number of blocks that have published their partial max
+    uint32_t ticket;  // number of slot groups whose last block has arrived
     uint32_t pad0[31];
     struct {
-        uint32_t bits;  // running max of |x| as an unsigned bit pattern (NaN patterns compare above Inf)
-        uint32_t pad[31];
+        uint32_t bits;    // running max of |x| as an unsigned bit pattern (NaN patterns compare above Inf)
+        uint32_t ticket;  // number of blocks of this slot's group (blockIdx % kMaxSlots) that have published
+        uint32_t pad[30];
     } slot[kMaxSlots];
     uint32_t pad1[(NTFP8_WORKSPACE_BYTES - 128 - 128 * kMaxSlots) / 4];
 };

@@ -151,11 +151,21 @@ __device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, c
         uint32_t bm = 0;
 #pragma unroll
         for (int i = 0; i < THREADS / 64; ++i) bm = s_part[i] > bm ? s_part[i] : bm;
-        const uint32_t old = __hip_atomic_fetch_max(&ws->slot[blockIdx.x % kMaxSlots].bits, bm, __ATOMIC_RELAXED,
-                                                    __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("s_waitcnt vmcnt(0)" ::"v"(old) : "memory");
-        const uint32_t t = __hip_atomic_fetch_add(&ws->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (t == gridDim.x - 1);
+        // Two-level arrival count: a block publishes into the slot of its group and draws a ticket there; the
+        // last block of a group draws a ticket of the launch.  All blocks finish at about the same time, and
+        // their atomics on one address would queue one behind the other.
+        const uint32_t grp = blockIdx.x % kMaxSlots;
+        const uint32_t old = __hip_atomic_fetch_max(&ws->slot[grp].bits, bm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::"v"(old) : "memory");   // the max is in place before the ticket is drawn
+        const uint32_t in_group = (gridDim.x - grp + kMaxSlots - 1) / kMaxSlots;
+        const uint32_t t = __hip_atomic_fetch_add(&ws->slot[grp].ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        bool last = false;
+        if (t == in_group - 1) {
+            const uint32_t groups = gridDim.x < (uint32_t)kMaxSlots ? gridDim.x : (uint32_t)kMaxSlots;
+            const uint32_t t2 = __hip_atomic_fetch_add(&ws->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last = (t2 == groups - 1);
+        }
+        s_last = last;
     }
     __syncthreads();
     // The epilogue runs on the first wave of the block that drew the last ticket: every global access
@@ -195,7 +205,10 @@ __device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, c
         if (io.hist) *io.scale_state = update_scale(__uint_as_float(hm), used, io.fmt, io.margin);
         __hip_atomic_store(&ws->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (lane < kMaxSlots) __hip_atomic_store(&ws->slot[lane].bits, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane < kMaxSlots) {
+        __hip_atomic_store(&ws->slot[lane].bits, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&ws->slot[lane].ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 
 __device__ __forceinline__ bool degenerate_scale(float s) {
