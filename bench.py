@@ -31,6 +31,12 @@ if ROOT not in sys.path:
 
 PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA peak
 PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E peak
+# HBM-side traffic measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (one counter per run, KiB per dispatch
+# scaled by what the same counter reads for a 128 MiB copy: x2.0 for FETCH_SIZE, x1.0 for WRITE_SIZE); the figures
+# and the commands are in profiles/hbm_traffic_counters.txt.  Bytes, summed over the GEMM launches of one step /
+# for one launch of the fused quantise kernel on the [4096,4096] bf16 tensor.
+GEMM_TRAFFIC_PER_STEP = {"fetch": 4201.6e6, "write": 1482.3e6}
+QUANT_TRAFFIC_PER_LAUNCH = {"fetch": 33.69e6, "write": 16.79e6}
 
 TOKENS = 4096
 LINEARS = [  # name, in_features (K), out_features (N)
@@ -103,6 +109,15 @@ def linear_step(mods, xs, gys, wstream=None):
         x.grad = None
         y = lin(x)
         y.backward(gy)
+
+
+def gemm_algorithmic_bytes():
+    """Operand bytes read once plus output bytes written once, summed over the 15 GEMMs of a step
+    (fp8 operands; bf16 outputs for forward and dgrad, fp32 for wgrad)."""
+    T, total = TOKENS, 0
+    for _, K, N in LINEARS:
+        total += (T * K + N * K + 2 * T * N) + (T * N + N * K + 2 * T * K) + (T * N + T * K + 4 * N * K)
+    return float(total)
 
 
 def gemm_in_step_timing(step, first_index, steps):
@@ -365,7 +380,10 @@ def main():
                        "tokens": TOKENS, "linears": [f"{n}:{k}->{o}" for n, k, o in LINEARS],
                        "flops_per_step": flops_step, "pct_fp8_peak": round(100 * value / PEAK_FP8_TFLOPS, 2)},
             "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(achieved / PEAK_FP8_TFLOPS, 4), "traffic": None,
+                         "frac": round(achieved / PEAK_FP8_TFLOPS, 4),
+                         "traffic": GEMM_TRAFFIC_PER_STEP["fetch"] + GEMM_TRAFFIC_PER_STEP["write"],
+                         "traffic_unit": "bytes per step, all GEMM launches (fetch + write counters)",
+                         "algorithmic_bytes": gemm_algorithmic_bytes(),
                          "kernel": "gemm_nt_big_kernel", "timing": "HIP events around every GEMM call inside the step",
                          "gemm_ms_per_step": round(gms, 4), "calls": per_call},
         })
@@ -381,7 +399,8 @@ def main():
                         "ms": {k: round(v, 5) for k, v in qms.items()},
                         "roofline": {"bound": "hbm", "achieved": round(qb / (q_avg * 1e-3) / 1e9, 1),
                                      "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                                     "frac": round(qb / (q_avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4), "traffic": None}}
+                                     "frac": round(qb / (q_avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+                                     "traffic": sum(QUANT_TRAFFIC_PER_LAUNCH.values()), "algorithmic_bytes": qb}}
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_baseline_linear()
     else:
@@ -394,7 +413,8 @@ def main():
             "config": {"workload": "bf16 [4096,4096] delayed-scaling quantise, e4m3 + e5m2 per step, hist 16",
                        "bytes_per_step": bytes_step, "pct_hbm_peak": round(100 * value / PEAK_HBM_GBPS, 2)},
             "roofline": {"bound": "hbm", "achieved": round(qb / (q_avg * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBPS,
-                         "unit": "GB/s", "frac": round(qb / (q_avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4), "traffic": None,
+                         "unit": "GB/s", "frac": round(qb / (q_avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+                         "traffic": sum(QUANT_TRAFFIC_PER_LAUNCH.values()), "algorithmic_bytes": qb,
                          "kernel": "quant_flat_kernel", "ms": {k: round(v, 5) for k, v in qms.items()}},
         })
         if not args.no_cpu_baseline:
