@@ -4,20 +4,20 @@
 // SIMD.  Each wave owns (16 MI) x 128 outputs as MI x 8 accumulator blocks of V_MFMA_F32_16X16X128_F8F6F4
 // (MI = 8: 256-row block tile, 256 accumulator registers per lane; MI = 4: 128-row block tile).
 //
-// Data movement per K-tile: every wave brings a quarter of the A and B tiles from global memory
-// straight into LDS (16 bytes per lane, XOR-swizzled), reads its MI A fragments from LDS once and
-// keeps them in registers, and streams its 8 B fragments from LDS two MFMA groups ahead of their
-// use.  One MFMA group = the MI MFMAs that share one B fragment.
+// Data movement per K-tile: every wave brings a quarter of the A and B tiles from global memory into
+// LDS (16 bytes per lane, XOR-swizzled), reads its MI A fragments from LDS once and keeps them in
+// registers, and streams its 8 B fragments from LDS two MFMA groups ahead of their use.  One MFMA
+// group = the MI MFMAs that share one B fragment.
 //
 // Pipeline, two LDS stages, ONE workgroup barrier per K-tile placed after MFMA group 5:
-//   * before the barrier a wave has read every fragment of the current tile into registers, so after
-//     it the current stage can be refilled with tile kt + 2 (first half of the loads under groups
-//     6-7, second half under groups 0-1 of the next tile);
-//   * the barrier also publishes tile kt + 1 (each wave waits for its own loads first).  Groups 6 and 7
-//     are issued interleaved, two MFMAs per A fragment; the fragment register is dead after them and is
-//     refilled on the spot with the same fragment of tile kt + 1, so one set of A registers suffices.
-// The matrix pipe therefore never waits for LDS or for the barrier's stragglers by more than the
-// skew between waves, and the loads of a tile have more than a full tile of MFMA time to land.
+//   * before the barrier a wave has read every fragment of the current tile into registers, so the
+//     barrier releases the current stage for tile kt + 2 and publishes tile kt + 1 at once;
+//   * groups 6 and 7 are issued interleaved, two MFMAs per A fragment; the fragment register is dead
+//     after them and is refilled with the same fragment of tile kt + 1, so one set of A registers
+//     suffices.
+// Global loads: whole tiles (MI = 8) keep one K-tile in flight in registers and write it to LDS a
+// K-tile later, so that every load has a full K-tile of MFMA time to arrive; half tiles (MI = 4) have
+// no registers to spare and load straight into the released LDS stage.
 #pragma once
 
 namespace ntfp8 {
