@@ -9,7 +9,7 @@ from nanotron_amd.fp8.dtypes import DTypes
 from nanotron_amd.fp8.kernel import fp8_matmul_kernel
 from nanotron_amd.fp8.meta import FP8Meta
 from nanotron_amd.fp8.parameter import FP8Parameter
-from nanotron_amd.fp8.tensor import DelayedScaling, FP8Tensor, update_scaling_factor
+from nanotron_amd.fp8.tensor import DelayedScaling, FP8Tensor, cast_with_scale, update_scaling_factor
 
 
 class FP8LinearMeta(TypedDict):
@@ -91,6 +91,58 @@ class FP8Linear(nn.Linear):
             t.record_stream(cur)
         w.data = q
         self._weight_ready = ready
+
+    # ---- checkpoints -------------------------------------------------------------------------------
+    # The reference serialises no FP8 state (nothing under src/nanotron/serialize knows about it).  Here a
+    # layer with delayed scaling adds four fp32 tensors to its state dict, `fp8_state.<role>` =
+    # [seen a usable amax (0/1), scale for the next step, amax history newest first] and
+    # `fp8_state.weight_scale` = the scale the current fp8 weight copy was cast with, so that a resumed run
+    # continues the delayed-scaling trajectory bit for bit.  Layers without delayed scaling add nothing, and
+    # a state dict without these keys loads as before.
+    _FP8_STATE = "fp8_state."
+
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        super()._save_to_state_dict(destination, prefix, keep_vars)
+        if self.scaling is None:
+            return
+        for role, st in self.scaling.items():
+            flag = torch.tensor([1.0 if st.initialised else 0.0], dtype=torch.float32, device=st._buf.device)
+            destination[prefix + self._FP8_STATE + role] = torch.cat([flag, st._buf.detach()])
+        destination[prefix + self._FP8_STATE + "weight_scale"] = self.weight.fp8_meta.scale.detach().reshape(1).clone()
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs):
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys, error_msgs)
+        mine = {k: v for k, v in state_dict.items() if k.startswith(prefix + self._FP8_STATE)}
+        for k in mine:
+            if k in unexpected_keys:
+                unexpected_keys.remove(k)
+        if not isinstance(self.weight, FP8Parameter):
+            return
+        weight_scale = None
+        if self.scaling is not None:
+            for role, st in self.scaling.items():
+                t = mine.get(prefix + self._FP8_STATE + role)
+                if t is None:
+                    if strict:
+                        missing_keys.append(prefix + self._FP8_STATE + role)
+                    continue
+                if t.numel() != 2 + st.history_len:
+                    error_msgs.append(f"{prefix}{self._FP8_STATE}{role}: amax history of length {t.numel() - 2}, "
+                                      f"this layer keeps {st.history_len}")
+                    continue
+                t = t.to(device=st._buf.device, dtype=torch.float32)
+                st._buf.copy_(t[1:])
+                st.initialised = bool(t[0].item() != 0.0)
+            weight_scale = mine.get(prefix + self._FP8_STATE + "weight_scale")
+        # the master weight has just been overwritten: rebuild the fp8 copy (and its transpose) from it
+        w = self.weight
+        hp = w.as_subclass(torch.Tensor)
+        with torch.no_grad():
+            if weight_scale is not None:
+                w.data = cast_with_scale(hp, weight_scale, DTypes.FP8E4M3, with_transpose=True)
+            else:
+                w.data = FP8Tensor(hp, dtype=DTypes.FP8E4M3, with_transpose=True)
+        self._weight_ready = None
 
     def forward(self, input: Union[FP8Tensor, torch.Tensor]) -> torch.Tensor:
         # fp8 kernels only when both input and weight are on the GPU (linear.py:53-54)

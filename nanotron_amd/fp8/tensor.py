@@ -163,6 +163,38 @@ def _quantize(cls, tensor: torch.Tensor, dtype: DTypes, state: Optional[DelayedS
     return obj
 
 
+def cast_with_scale(tensor: torch.Tensor, scale: torch.Tensor, dtype: DTypes, with_transpose: bool = False) -> FP8Tensor:
+    """FP8Tensor of `tensor` cast with a given device scale (no amax pass, no delayed-scaling state touched):
+    the cast half of the reference's FP8Tensor.__new__ (src/nanotron/fp8/tensor.py:28,60-65).  Used to
+    rebuild an fp8 copy exactly as it was, e.g. after loading a checkpoint."""
+    from nanotron_amd.fp8.meta import FP8Meta
+
+    x = tensor.detach()
+    if not x.is_contiguous():
+        x = x.contiguous()
+    dev = x.device
+    assert dev != torch.device("cpu"), "cast_with_scale only supports CUDA tensors"
+    cols = x.shape[-1] if x.dim() >= 2 else x.numel()
+    rows = x.numel() // cols
+    scalars = torch.zeros(2, dtype=torch.float32, device=dev)  # [amax (not computed), scale]
+    scalars[1].copy_(scale.reshape(()).to(device=dev, dtype=torch.float32))
+    out = torch.empty(x.shape, dtype=torch.uint8, device=dev)
+    out_t = None
+    if with_transpose:
+        assert x.dim() == 2, "with_transpose needs a 2-D tensor"
+        out_t = torch.empty((cols, rows), dtype=torch.uint8, device=dev)
+    nt.check(nt.lib.ntfp8_cast_to_fp8(x.data_ptr(), nt.TORCH_TO_NT[x.dtype], rows, cols, scalars[1].data_ptr(), _FMT[dtype],
+                                      out.data_ptr(), nt.ptr(out_t), nt.stream_ptr(dev)), "ntfp8_cast_to_fp8")
+    meta = FP8Meta(scalars[0], scalars[1], dtype)
+    obj = torch.Tensor._make_subclass(FP8Tensor, out)
+    obj.fp8_meta = meta
+    if out_t is not None:
+        t = torch.Tensor._make_subclass(FP8Tensor, out_t)
+        t.fp8_meta = meta
+        obj._transposed = t
+    return obj
+
+
 def convert_torch_dtype_to_te_dtype(dtype) -> DType:
     """Reference: src/nanotron/fp8/tensor.py:39-55 (same key set, returns this library's enum)."""
     mapping = {
