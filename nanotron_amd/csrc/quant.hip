@@ -140,8 +140,26 @@ __device__ __forceinline__ uint8_t encode1(float x, float scale) {
 // XCDs agree) and orders them with the wave's own memory counter: the partial max is folded in with
 // a returning atomic, the wave waits for it, then takes a ticket.  A release fence here would write
 // back the whole L2 once per block, which costs more than the streaming pass itself.
+// What the last block's epilogue will read, requested by the first wave of every block while the
+// tensor is still streaming: the history entry that moves into this lane's slot and the scale in
+// force.  It takes one round trip out of the dependent chain at the end of the kernel.
+struct EpiloguePrefetch {
+    float hist_prev;  // hist[lane - 1] (lanes 1 .. hist_len-1; histories of up to 64 entries)
+    float scale;      // *scale_state
+};
+__device__ __forceinline__ EpiloguePrefetch prefetch_epilogue(const ScalarIO& io, int mode) {
+    EpiloguePrefetch p = {0.0f, 1.0f};
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        if (io.hist && io.hist_len <= 64 && lane >= 1 && lane < io.hist_len) p.hist_prev = io.hist[lane - 1];
+        if (mode != kModeAmaxOnly) p.scale = *io.scale_state;
+    }
+    return p;
+}
+
 template <int THREADS>
-__device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, const ScalarIO& io, int mode) {
+__device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, const ScalarIO& io, int mode,
+                                            const EpiloguePrefetch& pre) {
     __shared__ uint32_t s_part[THREADS / 64];
     __shared__ bool s_last;
     const uint32_t wm = wave_max_u32(m_f32bits);
@@ -182,10 +200,17 @@ __device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, c
         const float old = io.old_scale ? *io.old_scale : 1.0f;
         used = update_scale(a, old, io.fmt, io.margin);
     } else {
-        used = *io.scale_state;
+        used = pre.scale;
     }
     uint32_t hm = bits;
-    if (io.hist) {
+    if (io.hist && io.hist_len <= 64) {
+        const bool ok = lane < io.hist_len;
+        const float h = lane == 0 ? a : pre.hist_prev;
+        if (ok) io.hist[lane] = h;
+        const uint32_t hb = wave_max_u32(ok ? (__float_as_uint(h) & 0x7fffffffu) : 0u);
+        hm = hb > hm ? hb : hm;
+        if (hm > kInfBits) hm = kNanBits;
+    } else if (io.hist) {
         // hist[i] <- hist[i-1], hist[0] <- a; 64 entries per trip, highest chunk first so that an entry is
         // read before the chunk below overwrites it
         for (int base = ((io.hist_len - 1) / 64) * 64; base >= 0; base -= 64) {
@@ -232,6 +257,8 @@ __global__ __launch_bounds__(kFlatThreads) void quant_flat_kernel(const typename
         scale = *scale_ptr;
         degen = degenerate_scale(scale);
     }
+    EpiloguePrefetch pre = {0.0f, 1.0f};
+    if constexpr (kAmax) pre = prefetch_epilogue(io, MODE);
     uint32_t m_run = 0;  // in source-format bits
     const int64_t stride = (int64_t)gridDim.x * kFlatThreads;
     int64_t i = (int64_t)blockIdx.x * kFlatThreads + threadIdx.x;
@@ -269,7 +296,7 @@ __global__ __launch_bounds__(kFlatThreads) void quant_flat_kernel(const typename
         if constexpr (kAmax) m_run = m > m_run ? m : m_run;
         if constexpr (kCast) out[j] = encode1<F>(xv, scale);
     }
-    if constexpr (kAmax) publish_and_finalize<kFlatThreads>(L::to_f32_bits(m_run), ws, io, MODE);
+    if constexpr (kAmax) publish_and_finalize<kFlatThreads>(L::to_f32_bits(m_run), ws, io, MODE, pre);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -296,6 +323,8 @@ __global__ __launch_bounds__(kTileThreads) void quant_transpose_kernel(const typ
     const int cchunk = t & 7;   // 16-column chunk inside the tile
     const int rsub = t >> 3;    // 0..31
     const int rchunk = t & 7;
+    EpiloguePrefetch pre = {0.0f, 1.0f};
+    if constexpr (kAmax) pre = prefetch_epilogue(io, kModeDelayed);
     uint32_t m_run = 0;
     // persistent over tiles: the number of blocks (and so of reduction atomics) stays ~2 per CU
     for (int64_t tile_id = blockIdx.x; tile_id < tiles; tile_id += gridDim.x) {
@@ -326,7 +355,7 @@ __global__ __launch_bounds__(kTileThreads) void quant_transpose_kernel(const typ
     }
     __syncthreads();  // the tile buffer is reused by the next trip
     }
-    if constexpr (kAmax) publish_and_finalize<kTileThreads>(L::to_f32_bits(m_run), ws, io, kModeDelayed);
+    if constexpr (kAmax) publish_and_finalize<kTileThreads>(L::to_f32_bits(m_run), ws, io, kModeDelayed, pre);
 }
 
 // Any shape: one element per thread step, transposed store.  Used when the tile kernel's
@@ -339,6 +368,8 @@ __global__ __launch_bounds__(kThreads) void quant_transpose_scalar_kernel(
     const float scale = *scale_ptr;
     const int64_t n = rows * cols;
     const int64_t stride = (int64_t)gridDim.x * kThreads;
+    EpiloguePrefetch pre = {0.0f, 1.0f};
+    if constexpr (kAmax) pre = prefetch_epilogue(io, kModeDelayed);
     uint32_t m_run = 0;
     for (int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x; j < n; j += stride) {
         uint32_t m;
@@ -349,7 +380,7 @@ __global__ __launch_bounds__(kThreads) void quant_transpose_scalar_kernel(
         const int64_t r = j / cols, c = j % cols;
         out_t[c * rows + r] = b;
     }
-    if constexpr (kAmax) publish_and_finalize<kThreads>(L::to_f32_bits(m_run), ws, io, kModeDelayed);
+    if constexpr (kAmax) publish_and_finalize<kThreads>(L::to_f32_bits(m_run), ws, io, kModeDelayed, pre);
 }
 
 // ---------------------------------------------------------------------------------------------
