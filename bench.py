@@ -122,42 +122,50 @@ def gemm_algorithmic_bytes():
 
 def gemm_in_step_timing(step, first_index, steps):
     """Times every GEMM call where it runs: `steps` further steps of the same workload with a HIP event
-    recorded on the launch stream before and after each call of the GEMM entry point.  Returns
-    (flops, milliseconds) summed over one step and the per-call averages in call order."""
+    recorded on the launch stream before and after each call of the GEMM entry points (a backward issues
+    its dgrad and wgrad as one batched call).  Returns (flops, milliseconds) summed over one step and the
+    per-call averages in call order."""
     import torch
 
     from nanotron_amd.fp8 import kernel as K
 
-    orig = K._gemm_nt
+    orig_one, orig_batch = K._gemm_nt, K._gemm_nt_batch
     log = []
 
-    def timed(a, b, out_dtype, accumulate_into):
+    def bracket(fn, shapes):
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         e0.record()
-        out = orig(a, b, out_dtype, accumulate_into)
+        out = fn()
         e1.record()
-        log.append((a.shape[0], b.shape[0], a.shape[1], e0, e1))
+        log.append((shapes, e0, e1))
         return out
 
-    K._gemm_nt = timed
+    def timed_one(a, b, out_dtype, accumulate_into):
+        return bracket(lambda: orig_one(a, b, out_dtype, accumulate_into), [(a.shape[0], b.shape[0], a.shape[1])])
+
+    def timed_batch(problems):
+        return bracket(lambda: orig_batch(problems), [(p[0].shape[0], p[1].shape[0], p[0].shape[1]) for p in problems])
+
+    K._gemm_nt, K._gemm_nt_batch = timed_one, timed_batch
     try:
         for i in range(steps):
             step(first_index + i)
         torch.cuda.synchronize()
     finally:
-        K._gemm_nt = orig
+        K._gemm_nt, K._gemm_nt_batch = orig_one, orig_batch
     per_step = len(log) // steps
-    names = [f"{n}.{t}" for n, _, _ in LINEARS for t in ("fwd", "dgrad", "wgrad")]
+    names = [f"{n}.{t}" for n, _, _ in LINEARS for t in ("fwd", "dgrad+wgrad")]
     assert per_step == len(names), (per_step, len(names))
     total_flops, total_ms, per_call = 0.0, 0.0, []
     for c in range(per_step):
-        M, N, Kd = log[c][:3]
-        ms = sum(log[s * per_step + c][3].elapsed_time(log[s * per_step + c][4]) for s in range(steps)) / steps
-        flops = 2.0 * M * N * Kd
+        shapes = log[c][0]
+        ms = sum(log[s * per_step + c][1].elapsed_time(log[s * per_step + c][2]) for s in range(steps)) / steps
+        flops = sum(2.0 * M * N * Kd for M, N, Kd in shapes)
         total_flops += flops
         total_ms += ms
-        per_call.append({"gemm": names[c], "mnk": [M, N, Kd], "ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1)})
+        per_call.append({"gemm": names[c], "mnk": [list(x) for x in shapes], "ms": round(ms, 4),
+                         "tflops": round(flops / ms / 1e9, 1)})
     return total_flops, total_ms, per_call
 
 

@@ -112,6 +112,23 @@ int ntfp8_gemm(const void* A, int fmt_a, const float* scale_a,
                const void* B, int fmt_b, const float* scale_b,
                void* D, int d_dtype, int64_t M, int64_t N, int64_t K, int accumulate, void* stream);
 
+/* Several independent GEMMs in one call: no output may overlap an operand or output of another
+ * problem.  Problems with the same operand formats share launches, which removes the partial last
+ * round of tiles and the kernel boundary between them.  The reference issues the dgrad and wgrad of
+ * a layer as two tex.te_gemm calls on the same stream (src/nanotron/fp8/linear.py:104-109); they
+ * do not depend on each other.  Each problem means what it means for ntfp8_gemm. */
+typedef struct ntfp8_gemm_desc {
+    const void* A;
+    const float* scale_a;
+    const void* B;
+    const float* scale_b;
+    void* D;
+    int64_t M, N, K;
+    int fmt_a, fmt_b, d_dtype, accumulate;
+} ntfp8_gemm_desc;
+#define NTFP8_MAX_BATCH 64
+int ntfp8_gemm_batch(const ntfp8_gemm_desc* problems, int count, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

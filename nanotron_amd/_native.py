@@ -31,6 +31,13 @@ _lib = ctypes.CDLL(LIB_PATH)
 _c = ctypes
 _vp, _i, _i64, _f = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_float
 
+class GemmDesc(ctypes.Structure):
+    """`ntfp8_gemm_desc` of include/ntfp8.h."""
+    _fields_ = [("A", _vp), ("scale_a", _vp), ("B", _vp), ("scale_b", _vp), ("D", _vp),
+                ("M", _i64), ("N", _i64), ("K", _i64),
+                ("fmt_a", _i), ("fmt_b", _i), ("d_dtype", _i), ("accumulate", _i)]
+
+
 SIGNATURES = {
     "ntfp8_version": (_i, []),
     "ntfp8_strerror": (_c.c_char_p, [_i]),
@@ -43,6 +50,7 @@ SIGNATURES = {
     "ntfp8_cast_from_fp8": (_i, [_vp, _i, _vp, _i64, _vp, _i, _vp]),
     "ntfp8_transpose": (_i, [_vp, _i64, _i64, _vp, _vp]),
     "ntfp8_gemm": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i64, _i64, _i64, _i, _vp]),
+    "ntfp8_gemm_batch": (_i, [_c.POINTER(GemmDesc), _i, _vp]),
 }
 
 for _name, (_res, _args) in SIGNATURES.items():

@@ -10,8 +10,8 @@ int run_dequant(const void* in, int fmt, const float* scale, int64_t n, void* ou
 int run_transpose(const void* in, int64_t rows, int64_t cols, void* out, hipStream_t st);
 int run_update_scale(const float* amax, const float* old_scale, int fmt, int margin, float* out, int64_t n,
                      hipStream_t st);
-int run_gemm(const void* A, int fmt_a, const float* sa, const void* B, int fmt_b, const float* sb, void* D, int d_dtype,
-             int M, int N, int K, int accumulate, hipStream_t st);
+int run_gemm(const GemmDesc& g, hipStream_t st);
+int run_gemm_batch(const GemmDesc* g, int n, hipStream_t st);
 
 namespace {
 
@@ -52,6 +52,24 @@ int check_outputs(const void* x, int x_dtype, int64_t n, const void* out, const 
     if (out && overlap(x, xb, out, (size_t)n)) return NTFP8_ERR_ALIAS;
     if (out_t && overlap(x, xb, out_t, (size_t)n)) return NTFP8_ERR_ALIAS;
     if (out && out_t && overlap(out, (size_t)n, out_t, (size_t)n)) return NTFP8_ERR_ALIAS;
+    return NTFP8_OK;
+}
+
+// argument checks of one GEMM problem; fills the launchers' descriptor
+int check_gemm(const ntfp8_gemm_desc& p, GemmDesc* g) {
+    if (!p.A || !p.B || !p.D || !p.scale_a || !p.scale_b) return NTFP8_ERR_NULL;
+    if (!fmt_ok(p.fmt_a) || !fmt_ok(p.fmt_b) || !dtype_ok(p.d_dtype)) return NTFP8_ERR_ENUM;
+    const int64_t M = p.M, N = p.N, K = p.K;
+    if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffff00LL || N > 0x7fffff00LL || K > 0x7fffff00LL) return NTFP8_ERR_SIZE;
+    int64_t mn, mk, nk;
+    if (!numel(M, N, &mn) || !numel(M, K, &mk) || !numel(N, K, &nk)) return NTFP8_ERR_SIZE;
+    if (((M + 127) / 128) * ((N + 127) / 128) > 0x7fffffffLL) return NTFP8_ERR_SIZE;
+    if (p.accumulate && p.d_dtype != NTFP8_F32) return NTFP8_ERR_UNSUPPORTED;
+    if (!is_aligned(p.scale_a, 4) || !is_aligned(p.scale_b, 4) || !is_aligned(p.D, dtype_size(p.d_dtype)))
+        return NTFP8_ERR_ALIGN;
+    const size_t db = (size_t)mn * dtype_size(p.d_dtype);
+    if (overlap(p.A, (size_t)mk, p.D, db) || overlap(p.B, (size_t)nk, p.D, db)) return NTFP8_ERR_ALIAS;
+    *g = GemmDesc{p.A, p.fmt_a, p.scale_a, p.B, p.fmt_b, p.scale_b, p.D, p.d_dtype, (int)M, (int)N, (int)K, p.accumulate ? 1 : 0};
     return NTFP8_OK;
 }
 
@@ -183,18 +201,33 @@ int ntfp8_transpose(const void* in, int64_t rows, int64_t cols, void* out, void*
 
 int ntfp8_gemm(const void* A, int fmt_a, const float* scale_a, const void* B, int fmt_b, const float* scale_b, void* D,
                int d_dtype, int64_t M, int64_t N, int64_t K, int accumulate, void* stream) {
-    if (!A || !B || !D || !scale_a || !scale_b) return NTFP8_ERR_NULL;
-    if (!fmt_ok(fmt_a) || !fmt_ok(fmt_b) || !dtype_ok(d_dtype)) return NTFP8_ERR_ENUM;
-    if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffff00LL || N > 0x7fffff00LL || K > 0x7fffff00LL) return NTFP8_ERR_SIZE;
-    int64_t mn, mk, nk;
-    if (!numel(M, N, &mn) || !numel(M, K, &mk) || !numel(N, K, &nk)) return NTFP8_ERR_SIZE;
-    if (((M + 127) / 128) * ((N + 127) / 128) > 0x7fffffffLL) return NTFP8_ERR_SIZE;
-    if (accumulate && d_dtype != NTFP8_F32) return NTFP8_ERR_UNSUPPORTED;
-    if (!is_aligned(scale_a, 4) || !is_aligned(scale_b, 4) || !is_aligned(D, dtype_size(d_dtype))) return NTFP8_ERR_ALIGN;
-    const size_t db = (size_t)mn * dtype_size(d_dtype);
-    if (overlap(A, (size_t)mk, D, db) || overlap(B, (size_t)nk, D, db)) return NTFP8_ERR_ALIAS;
-    return run_gemm(A, fmt_a, scale_a, B, fmt_b, scale_b, D, d_dtype, (int)M, (int)N, (int)K, accumulate,
-                    static_cast<hipStream_t>(stream));
+    const ntfp8_gemm_desc p = {A, scale_a, B, scale_b, D, M, N, K, fmt_a, fmt_b, d_dtype, accumulate};
+    GemmDesc g;
+    const int rc = check_gemm(p, &g);
+    if (rc) return rc;
+    return run_gemm(g, static_cast<hipStream_t>(stream));
+}
+
+int ntfp8_gemm_batch(const ntfp8_gemm_desc* problems, int count, void* stream) {
+    if (!problems) return NTFP8_ERR_NULL;
+    if (count <= 0 || count > NTFP8_MAX_BATCH) return NTFP8_ERR_SIZE;
+    GemmDesc g[NTFP8_MAX_BATCH];
+    for (int i = 0; i < count; ++i) {
+        const int rc = check_gemm(problems[i], &g[i]);
+        if (rc) return rc;
+    }
+    // independence: an output overlaps nothing of any other problem
+    for (int i = 0; i < count; ++i) {
+        const size_t di = (size_t)g[i].M * g[i].N * dtype_size(g[i].d_dtype);
+        for (int j = 0; j < count; ++j) {
+            if (i == j) continue;
+            const size_t dj = (size_t)g[j].M * g[j].N * dtype_size(g[j].d_dtype);
+            if (overlap(g[i].D, di, g[j].A, (size_t)g[j].M * g[j].K) || overlap(g[i].D, di, g[j].B, (size_t)g[j].N * g[j].K) ||
+                (i < j && overlap(g[i].D, di, g[j].D, dj)))
+                return NTFP8_ERR_ALIAS;
+        }
+    }
+    return run_gemm_batch(g, count, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -127,6 +127,20 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
     return v;
 }
 
+// one GEMM problem as the launchers see it (validated by the C entry points)
+struct GemmDesc {
+    const void* A;
+    int fmt_a;
+    const float* sa;
+    const void* B;
+    int fmt_b;
+    const float* sb;
+    void* D;
+    int d_dtype;
+    int M, N, K;
+    int accumulate;
+};
+
 // compute units of the current device (cached per device)
 inline int cu_count() {
     static int cached[64] = {0};

@@ -140,64 +140,124 @@ __global__ void gemm_nt_naive_kernel(const uint8_t* __restrict__ A, const uint8_
 // ---------------------------------------------------------------------------------------------
 enum GemmPath { kPathNaive = 0, kPathSmall = 1, kPathBig = 2 };
 
+// which kernel serves a problem
+static int path_of(const GemmDesc& g) {
+    const bool aligned16 = (g.K % 16 == 0) &&
+                           ((reinterpret_cast<uintptr_t>(g.A) | reinterpret_cast<uintptr_t>(g.B)) & 15) == 0 &&
+                           (reinterpret_cast<uintptr_t>(g.D) & 15) == 0;
+    if (!aligned16) return kPathNaive;
+    // the big kernel addresses its operands with 32-bit buffer offsets and wants enough tiles to matter
+    const bool fits32 = (int64_t)(g.M + 256) * g.K < (1LL << 31) && (int64_t)(g.N + kBigN) * g.K < (1LL << 31);
+    const bool worth = g.M > kBM && g.N > kBN && g.K >= 2 * kBK;
+    return (fits32 && worth) ? kPathBig : kPathSmall;
+}
+
+// One launch (plus one for the half-tile tail) of the big kernel over up to kBigMaxProblems problems of the
+// same operand formats.  Tiles are listed problem by problem, longest K first: the long tiles start together and
+// the shorter ones fill the rounds behind them.
+template <int FA, int FB>
+static int launch_big(const GemmDesc* const* g, int n, hipStream_t st) {
+    int order[kBigMaxProblems];
+    for (int i = 0; i < n; ++i) order[i] = i;
+    for (int i = 1; i < n; ++i)   // insertion sort, stable, K descending
+        for (int j = i; j > 0 && g[order[j]]->K > g[order[j - 1]]->K; --j) {
+            const int t = order[j];
+            order[j] = order[j - 1];
+            order[j - 1] = t;
+        }
+    BigLaunch L = {};
+    L.count = n;
+    int tiles = 0;
+    for (int i = 0; i < n; ++i) {
+        const GemmDesc& d = *g[order[i]];
+        BigProblem& p = L.p[i];
+        p.A = static_cast<const uint8_t*>(d.A);
+        p.B = static_cast<const uint8_t*>(d.B);
+        p.D = d.D;
+        p.scale_a = d.sa;
+        p.scale_b = d.sb;
+        p.M = d.M;
+        p.N = d.N;
+        p.K = d.K;
+        p.tiles_m = (d.M + 255) / 256;
+        p.tiles_n = (d.N + kBigN - 1) / kBigN;
+        p.tile_begin = tiles;
+        p.d_dtype = d.d_dtype;
+        p.accumulate = d.accumulate;
+        tiles += p.tiles_m * p.tiles_n;
+    }
+    const int rem = tiles % cu_count();
+    L.tail_tiles = (rem != 0 && 2 * rem <= cu_count()) ? rem : 0;
+    L.full_blocks = tiles - L.tail_tiles;
+    L.round_size = cu_count();
+    if (L.full_blocks > 0)
+        hipLaunchKernelGGL((gemm_nt_big_kernel<FA, FB, 8>), dim3(L.full_blocks), dim3(kBigThreads), 0, st, L);
+    if (L.tail_tiles > 0)
+        hipLaunchKernelGGL((gemm_nt_big_kernel<FA, FB, 4>), dim3(2 * L.tail_tiles), dim3(kBigThreads), 0, st, L);
+    return hipGetLastError() == hipSuccess ? NTFP8_OK : NTFP8_ERR_LAUNCH;
+}
+
 template <int FA, int FB, int DT, bool kAcc>
-static int launch_gemm(const void* A, const float* sa, const void* B, const float* sb, void* D, int M, int N, int K,
-                       int path, hipStream_t st) {
-    const uint8_t* a = static_cast<const uint8_t*>(A);
-    const uint8_t* b = static_cast<const uint8_t*>(B);
-    if (path == kPathBig) {
-        BigGrid g;
-        g.tiles_m = (M + 255) / 256;
-        g.tiles_n = (N + kBigN - 1) / kBigN;
-        const int tiles = g.tiles_m * g.tiles_n;
-        const int rem = tiles % cu_count();
-        g.tail_tiles = (rem != 0 && 2 * rem <= cu_count()) ? rem : 0;
-        g.full_blocks = tiles - g.tail_tiles;
-        if (g.full_blocks > 0)
-            hipLaunchKernelGGL((gemm_nt_big_kernel<FA, FB, DT, kAcc, 8>), dim3(g.full_blocks), dim3(kBigThreads), 0, st, a, b,
-                               D, sa, sb, M, N, K, g);
-        if (g.tail_tiles > 0)
-            hipLaunchKernelGGL((gemm_nt_big_kernel<FA, FB, DT, kAcc, 4>), dim3(2 * g.tail_tiles), dim3(kBigThreads), 0, st, a,
-                               b, D, sa, sb, M, N, K, g);
-    } else if (path == kPathSmall) {
-        const int tm = (M + kBM - 1) / kBM, tn = (N + kBN - 1) / kBN;
-        hipLaunchKernelGGL((gemm_nt_kernel<FA, FB, DT, kAcc>), dim3(tm * tn), dim3(kGemmThreads), 0, st, a, b, D, sa, sb,
-                           M, N, K, tm, tn);
+static int launch_small(const GemmDesc& g, int path, hipStream_t st) {
+    const uint8_t* a = static_cast<const uint8_t*>(g.A);
+    const uint8_t* b = static_cast<const uint8_t*>(g.B);
+    if (path == kPathSmall) {
+        const int tm = (g.M + kBM - 1) / kBM, tn = (g.N + kBN - 1) / kBN;
+        hipLaunchKernelGGL((gemm_nt_kernel<FA, FB, DT, kAcc>), dim3(tm * tn), dim3(kGemmThreads), 0, st, a, b, g.D, g.sa,
+                           g.sb, g.M, g.N, g.K, tm, tn);
     } else {
-        const int64_t blocks = ((int64_t)M * N + 255) / 256;
-        hipLaunchKernelGGL((gemm_nt_naive_kernel<FA, FB, DT, kAcc>), dim3((int)blocks), dim3(256), 0, st, a, b, D, sa, sb,
-                           M, N, K);
+        const int64_t blocks = ((int64_t)g.M * g.N + 255) / 256;
+        hipLaunchKernelGGL((gemm_nt_naive_kernel<FA, FB, DT, kAcc>), dim3((int)blocks), dim3(256), 0, st, a, b, g.D, g.sa,
+                           g.sb, g.M, g.N, g.K);
     }
     return hipGetLastError() == hipSuccess ? NTFP8_OK : NTFP8_ERR_LAUNCH;
 }
 
 template <int FA, int FB>
-static int dispatch_out(const void* A, const float* sa, const void* B, const float* sb, void* D, int d_dtype, int M,
-                        int N, int K, int accumulate, int path, hipStream_t st) {
-    if (d_dtype == NTFP8_F32)
-        return accumulate ? launch_gemm<FA, FB, NTFP8_F32, true>(A, sa, B, sb, D, M, N, K, path, st)
-                          : launch_gemm<FA, FB, NTFP8_F32, false>(A, sa, B, sb, D, M, N, K, path, st);
-    if (d_dtype == NTFP8_BF16) return launch_gemm<FA, FB, NTFP8_BF16, false>(A, sa, B, sb, D, M, N, K, path, st);
-    return launch_gemm<FA, FB, NTFP8_F16, false>(A, sa, B, sb, D, M, N, K, path, st);
+static int dispatch_fmt(const GemmDesc* const* g, int n, int path, hipStream_t st) {
+    if (path == kPathBig) return launch_big<FA, FB>(g, n, st);
+    const GemmDesc& d = *g[0];   // the small kernels take one problem
+    if (d.d_dtype == NTFP8_F32)
+        return d.accumulate ? launch_small<FA, FB, NTFP8_F32, true>(d, path, st)
+                            : launch_small<FA, FB, NTFP8_F32, false>(d, path, st);
+    if (d.d_dtype == NTFP8_BF16) return launch_small<FA, FB, NTFP8_BF16, false>(d, path, st);
+    return launch_small<FA, FB, NTFP8_F16, false>(d, path, st);
 }
 
-int run_gemm(const void* A, int fmt_a, const float* sa, const void* B, int fmt_b, const float* sb, void* D, int d_dtype,
-             int M, int N, int K, int accumulate, hipStream_t st) {
-    const bool aligned16 = (K % 16 == 0) &&
-                           ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 &&
-                           (reinterpret_cast<uintptr_t>(D) & 15) == 0;
-    int path = kPathNaive;
-    if (aligned16) {
-        // the big kernel addresses its operands with 32-bit buffer offsets and wants enough tiles to matter
-        const bool fits32 = (int64_t)(M + 256) * K < (1LL << 31) && (int64_t)(N + kBigN) * K < (1LL << 31);
-        const bool worth = M > kBM && N > kBN && K >= 2 * kBK;
-        path = (fits32 && worth) ? kPathBig : kPathSmall;
+static int dispatch(const GemmDesc* const* g, int n, int path, hipStream_t st) {
+    const int fa = g[0]->fmt_a, fb = g[0]->fmt_b;
+    if (fa == kE4M3) return fb == kE4M3 ? dispatch_fmt<kE4M3, kE4M3>(g, n, path, st) : dispatch_fmt<kE4M3, kE5M2>(g, n, path, st);
+    return fb == kE4M3 ? dispatch_fmt<kE5M2, kE4M3>(g, n, path, st) : dispatch_fmt<kE5M2, kE5M2>(g, n, path, st);
+}
+
+int run_gemm(const GemmDesc& g, hipStream_t st) {
+    const GemmDesc* one[1] = {&g};
+    return dispatch(one, 1, path_of(g), st);
+}
+
+// Independent problems (no output of one is an operand of another).  Problems that qualify for the big kernel
+// and share their operand formats go out together, up to kBigMaxProblems per launch; the rest one by one.
+int run_gemm_batch(const GemmDesc* g, int n, hipStream_t st) {
+    bool done[64] = {false};
+    if (n > 64) return NTFP8_ERR_SIZE;
+    for (int i = 0; i < n; ++i) {
+        if (done[i]) continue;
+        const GemmDesc* group[kBigMaxProblems];
+        int cnt = 0;
+        const int path = path_of(g[i]);
+        group[cnt++] = &g[i];
+        done[i] = true;
+        if (path == kPathBig) {
+            for (int j = i + 1; j < n && cnt < kBigMaxProblems; ++j)
+                if (!done[j] && g[j].fmt_a == g[i].fmt_a && g[j].fmt_b == g[i].fmt_b && path_of(g[j]) == kPathBig) {
+                    group[cnt++] = &g[j];
+                    done[j] = true;
+                }
+        }
+        const int rc = dispatch(group, cnt, path, st);
+        if (rc != NTFP8_OK) return rc;
     }
-    if (fmt_a == kE4M3)
-        return fmt_b == kE4M3 ? dispatch_out<kE4M3, kE4M3>(A, sa, B, sb, D, d_dtype, M, N, K, accumulate, path, st)
-                              : dispatch_out<kE4M3, kE5M2>(A, sa, B, sb, D, d_dtype, M, N, K, accumulate, path, st);
-    return fmt_b == kE4M3 ? dispatch_out<kE5M2, kE4M3>(A, sa, B, sb, D, d_dtype, M, N, K, accumulate, path, st)
-                          : dispatch_out<kE5M2, kE5M2>(A, sa, B, sb, D, d_dtype, M, N, K, accumulate, path, st);
+    return NTFP8_OK;
 }
 
 }  // namespace ntfp8

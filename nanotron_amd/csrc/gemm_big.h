@@ -140,41 +140,74 @@ __device__ __forceinline__ void store_wave_tile16(const v4f (&acc)[MI][NJ], void
 // whole by the MI = 8 kernel.  If the tile count leaves a partial last round over the CUs, the
 // remaining `tail_tiles` tiles are cut into two 128-row halves and computed by a second launch of
 // the MI = 4 kernel with 2 tail_tiles workgroups, so that the last round is half as long.
-struct BigGrid {
+//
+// One launch can carry several independent GEMMs of the same operand formats (the dgrad and wgrad of a
+// layer, say): their tiles form one list, longest K first, so that the rounds of one problem fill up
+// with tiles of the next instead of ending in a partial round and a kernel boundary each.
+struct BigProblem {
+    const uint8_t* A;
+    const uint8_t* B;
+    void* D;
+    const float* scale_a;
+    const float* scale_b;
+    int M, N, K;
     int tiles_m, tiles_n;   // 256 x 256 tiles
-    int full_blocks;        // tiles computed whole
-    int tail_tiles;         // tiles computed as two halves
+    int tile_begin;         // position of this problem's first tile in the launch's tile list
+    int d_dtype;            // NTFP8_F32 / NTFP8_F16 / NTFP8_BF16
+    int accumulate;         // fp32 outputs only: D += result
+};
+constexpr int kBigMaxProblems = 4;
+struct BigLaunch {
+    BigProblem p[kBigMaxProblems];
+    int count;
+    int full_blocks;        // tiles (of the whole list) computed whole
+    int tail_tiles;         // tiles at the end of the list computed as two halves
+    int round_size;         // workgroups resident at once: one per CU
 };
 
 // MI = 8 needs the whole register file of a SIMD for one wave (256 accumulators + fragments).  The
 // MI = 4 variant is held to half of it by declaring a launch bound of twice its real workgroup
 // size: given more registers than it needs, the compiler keeps its accumulators in a second
 // register set and copies them back and forth inside the K loop.
-template <int FA, int FB, int DT, bool kAcc, int MI>
+template <int FA, int FB, int MI>
 __global__ __launch_bounds__(MI == 8 ? kBigThreads : 2 * kBigThreads)
-void gemm_nt_big_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, void* __restrict__ Dv,
-                        const float* __restrict__ scale_a, const float* __restrict__ scale_b, int M, int N, int K,
-                        BigGrid g) {
+void gemm_nt_big_kernel(const BigLaunch L) {
     __shared__ __attribute__((aligned(1024))) uint8_t sA[2][32 * MI * kBK];
     __shared__ __attribute__((aligned(1024))) uint8_t sB[2][kBigN * kBK];
 
-    // ---- which tile (or half tile) is this workgroup's -------------------------------------------
+    // ---- which tile (or half tile) of which problem is this workgroup's ----------------------------
     int pid = blockIdx.x;
     int half = 0;
     if constexpr (MI == 8) {
-        if (g.full_blocks % kXcds == 0) pid = (pid % kXcds) * (g.full_blocks / kXcds) + pid / kXcds;
+        // Workgroups are dealt to the XCDs round robin.  Within each round of `round_size` workgroups (one per
+        // CU) an XCD gets a contiguous run of the tile list, so its L2 sees few operand panels; across rounds
+        // the list is walked in order, so that the long tiles at its head start together on the whole chip.
+        const int round0 = (pid / L.round_size) * L.round_size;
+        const int in_round = min(L.round_size, L.full_blocks - round0);
+        const int local = pid - round0;
+        if (in_round % kXcds == 0) pid = round0 + (local % kXcds) * (in_round / kXcds) + local / kXcds;
     } else {
-        const int nb = 2 * g.tail_tiles;
+        const int nb = 2 * L.tail_tiles;
         if (nb % kXcds == 0) pid = (pid % kXcds) * (nb / kXcds) + pid / kXcds;
         half = pid & 1;
-        pid = g.full_blocks + (pid >> 1);
+        pid = L.full_blocks + (pid >> 1);
     }
+    int which = 0;
+#pragma unroll
+    for (int i = 1; i < kBigMaxProblems; ++i)
+        if (i < L.count && pid >= L.p[i].tile_begin) which = i;
+    const BigProblem& P = L.p[which];
+    const uint8_t* __restrict__ A = P.A;
+    const uint8_t* __restrict__ B = P.B;
+    void* __restrict__ Dv = P.D;
+    const int M = P.M, N = P.N, K = P.K;
+    pid -= P.tile_begin;
     int pid_m, pid_n;
     {
-        const int in_group = kGroupM * g.tiles_n;
+        const int in_group = kGroupM * P.tiles_n;
         const int group = pid / in_group;
         const int first_m = group * kGroupM;
-        const int gsz = min(g.tiles_m - first_m, kGroupM);
+        const int gsz = min(P.tiles_m - first_m, kGroupM);
         pid_m = first_m + (pid % in_group) % gsz;
         pid_n = (pid % in_group) / gsz;
     }
@@ -196,7 +229,7 @@ void gemm_nt_big_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict
     const int ld_kc = ((lane & 7) ^ (lane >> 3) ^ (wave & 1)) << 4;
     // chunks of the last K-tile at k >= K must read as zero, not as the start of the next row
     const bool tail_dead = (KT - 1) * kBK + ld_kc >= K;
-    const float alpha = (1.0f / *scale_a) * (1.0f / *scale_b);
+    const float alpha = (1.0f / *P.scale_a) * (1.0f / *P.scale_b);
 
     {
         constexpr int LA = MI * 2 * 16 / 8 / kBigWaves;  // wave-level loads of the A tile per wave per stage
@@ -446,7 +479,16 @@ void gemm_nt_big_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict
         back(No{}, No{}, kt + 1);
         }
 
-        store_wave_tile16<DT, kAcc, MI, kBigNJ>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
+        // output type and accumulation are properties of the problem, not of the kernel
+        if (P.d_dtype == NTFP8_BF16) {
+            store_wave_tile16<NTFP8_BF16, false, MI, kBigNJ>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
+        } else if (P.d_dtype == NTFP8_F16) {
+            store_wave_tile16<NTFP8_F16, false, MI, kBigNJ>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
+        } else if (P.accumulate) {
+            store_wave_tile16<NTFP8_F32, true, MI, kBigNJ>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
+        } else {
+            store_wave_tile16<NTFP8_F32, false, MI, kBigNJ>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
+        }
     }
 }
 

@@ -33,6 +33,60 @@ def _gemm_nt(a: FP8Tensor, b: FP8Tensor, out_dtype: torch.dtype, accumulate_into
     return out
 
 
+def _gemm_nt_batch(problems):
+    """Several independent `_gemm_nt` problems, given as tuples (a, b, out_dtype, accumulate_into), in one call of
+    the library: GEMMs with the same operand formats share launches.  Returns the outputs in order."""
+    descs = (nt.GemmDesc * len(problems))()
+    outs, keep = [], []
+    dev = problems[0][0].device
+    for d, (a, b, out_dtype, accumulate_into) in zip(descs, problems):
+        assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[1], (tuple(a.shape), tuple(b.shape))
+        assert a.device == dev and b.device == dev
+        M, K = a.shape
+        N = b.shape[0]
+        if not a.is_contiguous():
+            a = a.contiguous()
+        if not b.is_contiguous():
+            b = b.contiguous()
+        ma, mb = a.fp8_meta, b.fp8_meta
+        if accumulate_into is not None:
+            assert accumulate_into.dtype == torch.float32 and accumulate_into.shape == (M, N)
+            assert accumulate_into.is_contiguous() and accumulate_into.device == dev
+            out, acc = accumulate_into, 1
+        else:
+            out, acc = torch.empty((M, N), dtype=out_dtype, device=dev), 0
+        d.A, d.scale_a, d.B, d.scale_b, d.D = a.data_ptr(), ma.scale.data_ptr(), b.data_ptr(), mb.scale.data_ptr(), out.data_ptr()
+        d.M, d.N, d.K = M, N, K
+        d.fmt_a, d.fmt_b, d.d_dtype, d.accumulate = _FMT[ma.dtype], _FMT[mb.dtype], nt.TORCH_TO_NT[out.dtype], acc
+        outs.append(out)
+        keep.append((a, b))
+    nt.check(nt.lib.ntfp8_gemm_batch(descs, len(problems), nt.stream_ptr(dev)), "ntfp8_gemm_batch")
+    return outs
+
+
+def _operands(mat_a: FP8Tensor, transpose_a: bool, mat_b: FP8Tensor, transpose_b: bool):
+    """(A, B) of the library's D = A . B^T for the reference's D = op_b(B) . op_a(A) (kernel.py:43-44)."""
+    assert mat_a.device != torch.device("cpu") and mat_b.device != torch.device("cpu"), \
+        "The tensors must be on a CUDA device in order to use the FP8 kernel!!"
+    assert hasattr(mat_a, "fp8_meta") and hasattr(mat_b, "fp8_meta"), "operands must be FP8Tensors"
+    a_ = mat_a if transpose_a else mat_a.transposed()
+    b_ = mat_b.transposed() if transpose_b else mat_b
+    return b_, a_
+
+
+@torch.no_grad()
+def fp8_matmul_pair(first: dict, second: dict):
+    """Two independent `fp8_matmul_kernel` calls (keyword dictionaries of its arguments) issued together, e.g. the
+    dgrad and wgrad of a layer (src/nanotron/fp8/linear.py:104-109 issues them one after the other).  Same
+    results as two calls; the library lets the two GEMMs share kernel launches."""
+    probs = []
+    for kw in (first, second):
+        A, B = _operands(kw["mat_a"], kw["transpose_a"], kw["mat_b"], kw["transpose_b"])
+        acc = kw.get("accumulate_into")
+        probs.append((A, B, (kw.get("out_dtype") or torch.float32) if acc is None else torch.float32, acc))
+    return _gemm_nt_batch(probs)
+
+
 @torch.no_grad()
 def fp8_matmul_kernel(
     mat_a: FP8Tensor,

@@ -6,7 +6,7 @@ from torch import nn
 
 from nanotron_amd.fp8.constants import INITIAL_AMAX, INITIAL_SCALING_FACTOR
 from nanotron_amd.fp8.dtypes import DTypes
-from nanotron_amd.fp8.kernel import fp8_matmul_kernel
+from nanotron_amd.fp8.kernel import fp8_matmul_kernel, fp8_matmul_pair
 from nanotron_amd.fp8.meta import FP8Meta
 from nanotron_amd.fp8.parameter import FP8Parameter
 from nanotron_amd.fp8.tensor import DelayedScaling, FP8Tensor, cast_with_scale, update_scaling_factor
@@ -203,29 +203,35 @@ class _FP8Matmul(torch.autograd.Function):
                                     with_transpose=weight.requires_grad)
 
         grad_input = None
-        if ctx.needs_input_grad[0]:
-            # dX[M,K] = dY[M,N] . W[N,K]
-            grad_input = fp8_matmul_kernel(
-                mat_a=weight.data, transpose_a=False, mat_b=grad_output, transpose_b=False, use_split_accumulator=True,
-                out_dtype=ctx.in_dtype or torch.float32,
-            )
-            if len(ctx.in_shape) != 2:
-                grad_input = grad_input.reshape(ctx.in_shape)
+        # dX[M,K] = dY[M,N] . W[N,K]
+        dgrad = dict(mat_a=weight.data, transpose_a=False, mat_b=grad_output, transpose_b=False, use_split_accumulator=True,
+                     out_dtype=ctx.in_dtype or torch.float32)
+        wgrad, slot = None, None
         if weight.requires_grad:
-            # dW[N,K] = dY[M,N]^T . X[M,K]
-            # The gradient is fp32 (kernel.py:24).  An fp32 parameter takes it as `.grad` (side effect, as
-            # linear.py:110); a 16-bit parameter cannot hold an fp32 `.grad`, so there it is kept beside the
-            # parameter as `.main_grad`, the fp32 master-gradient buffer an optimizer reads.
+            # dW[N,K] = dY[M,N]^T . X[M,K].  The gradient is fp32 (kernel.py:24).  An fp32 parameter takes it as `.grad`
+            # (side effect, as linear.py:110); a 16-bit parameter cannot hold an fp32 `.grad`, so there it is kept
+            # beside the parameter as `.main_grad`, the fp32 master-gradient buffer an optimizer reads.
             slot = "grad" if weight.dtype == torch.float32 else "main_grad"
             acc = None
             if module.accumulate_grad:
                 prev = getattr(weight, slot, None)
                 if prev is not None and prev.dtype == torch.float32:
                     acc = prev
-            grad_weight = fp8_matmul_kernel(
-                mat_a=input, transpose_a=False, mat_b=grad_output, transpose_b=True, use_split_accumulator=True,
-                accumulate_into=acc,
-            )
+            wgrad = dict(mat_a=input, transpose_a=False, mat_b=grad_output, transpose_b=True, use_split_accumulator=True,
+                         accumulate_into=acc)
+        grad_weight = None
+        if ctx.needs_input_grad[0] and wgrad is not None:
+            # the two GEMMs are independent: issued together they share kernel launches
+            grad_input, grad_weight = fp8_matmul_pair(
+                {k: v for k, v in dgrad.items() if k != "use_split_accumulator"},
+                {k: v for k, v in wgrad.items() if k != "use_split_accumulator"})
+        elif ctx.needs_input_grad[0]:
+            grad_input = fp8_matmul_kernel(**dgrad)
+        elif wgrad is not None:
+            grad_weight = fp8_matmul_kernel(**wgrad)
+        if grad_input is not None and len(ctx.in_shape) != 2:
+            grad_input = grad_input.reshape(ctx.in_shape)
+        if grad_weight is not None:
             setattr(weight, slot, grad_weight)
 
         return grad_input, None, None, None

@@ -214,3 +214,58 @@ def test_config3_and_4_llama7b_mlp_shapes():
     # dWd[H,I] = gd^T[H,M] . h[M,I]
     dwd = gpu_gemm_nt(gd.transposed(), h.transposed(), torch.float32).cpu()
     _sampled_rows_check(cpu(gd.transposed(), O.E5M2), cpu(h.transposed(), O.E4M3), dwd, torch.tensor([0, 77, 4095]))
+
+
+def test_batched_gemms_equal_separate_calls():
+    """ntfp8_gemm_batch: problems of one format pair share launches (their tiles form one list, longest K first),
+    others go out on their own; whatever the grouping, every output must equal the separate call bit for bit."""
+    from nanotron_amd.fp8.kernel import _gemm_nt_batch
+
+    def q(seed, shape, fmt, std=1.0):
+        return gpu_quant(O.normal_tensor(seed, shape, std), fmt, with_transpose=True)
+
+    x = q(1, (4096, 1024), O.E4M3)        # activations [M, K]
+    w = q(2, (1536, 1024), O.E4M3, 0.02)  # weight [N, K]
+    g = q(3, (4096, 1536), O.E5M2, 1e-3)  # output gradient [M, N]
+    small_a, small_b = q(4, (96, 160), O.E4M3), q(5, (80, 160), O.E4M3)
+    acc0 = O.normal_tensor(6, (1536, 1024), 1.0, torch.float32)
+    problems = [
+        (g, w.transposed(), torch.bfloat16, None),                  # dgrad  4096x1024x1536, e5m2 x e4m3
+        (g.transposed(), x.transposed(), torch.float32, None),      # wgrad  1536x1024x4096, e5m2 x e4m3, fp32
+        (x, w, torch.bfloat16, None),                               # fwd    4096x1536x1024, e4m3 x e4m3
+        (small_a, small_b, torch.float16, None),                    # served by the small kernel
+        (g.transposed(), x.transposed(), torch.float32, acc0.cuda()),  # wgrad accumulated into a master buffer
+        (g, w.transposed(), torch.float32, None),                   # a fifth e5m2 x e4m3 problem (> 4 per launch)
+        (g, w.transposed(), torch.float16, None),
+    ]
+    want = []
+    for a, b, dt, acc in problems:
+        want.append(gpu_gemm_nt(a, b, dt, None if acc is None else acc0.cuda()).cpu())
+    got = _gemm_nt_batch(problems)
+    assert len(got) == len(problems)
+    for (a, b, dt, acc), o, w_ in zip(problems, got, want):
+        assert o.dtype == (torch.float32 if acc is not None else dt)
+        if acc is not None:
+            assert o.data_ptr() == acc.data_ptr()
+        assert torch.equal(o.cpu(), w_)
+    # and against the oracle for the pair a backward issues
+    cpu = lambda t, fmt: O.Quantised(t.cpu().as_subclass(torch.Tensor), t.fp8_meta.amax.cpu(), t.fp8_meta.scale.cpu(), fmt)
+    dx = O.linear_dgrad(cpu(g, O.E5M2), cpu(w, O.E4M3), torch.bfloat16)
+    dw = O.linear_wgrad(cpu(g, O.E5M2), cpu(x, O.E4M3))
+    assert O.rel_l2(got[0].float().cpu(), dx.float()) <= 4e-3
+    assert O.rel_l2(got[1].cpu(), dw) <= REL_L2
+
+
+def test_batched_gemm_rejects_dependent_problems():
+    from nanotron_amd import _native as nt
+    from nanotron_amd.fp8.kernel import _gemm_nt_batch
+
+    a = gpu_quant(O.normal_tensor(11, (256, 256), 1.0), O.E4M3)
+    b = gpu_quant(O.normal_tensor(12, (256, 256), 1.0), O.E4M3)
+    out = torch.empty(256, 256, dtype=torch.float32, device="cuda")
+    with pytest.raises(RuntimeError):  # both problems write the same output
+        _gemm_nt_batch([(a, b, torch.float32, out), (b, a, torch.float32, out)])
+    descs = (nt.GemmDesc * 1)()
+    assert nt.lib.ntfp8_gemm_batch(descs, 0, None) == -3   # NTFP8_ERR_SIZE
+    assert nt.lib.ntfp8_gemm_batch(descs, 1, None) == -1   # NTFP8_ERR_NULL: empty descriptor
+    assert nt.lib.ntfp8_gemm_batch(None, 1, None) == -1
