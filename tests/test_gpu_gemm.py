@@ -269,3 +269,28 @@ def test_batched_gemm_rejects_dependent_problems():
     assert nt.lib.ntfp8_gemm_batch(descs, 0, None) == -3   # NTFP8_ERR_SIZE
     assert nt.lib.ntfp8_gemm_batch(descs, 1, None) == -1   # NTFP8_ERR_NULL: empty descriptor
     assert nt.lib.ntfp8_gemm_batch(None, 1, None) == -1
+
+
+def test_ragged_shapes_bit_exact_sweep():
+    """Seeded sweep over ragged shapes that take the large-tile kernels (edges in M and N, K tails of every
+    multiple of 16, odd and even K-tile counts, whole and half tiles), singly and as one batch."""
+    from nanotron_amd.fp8.kernel import _gemm_nt_batch
+
+    rng = torch.Generator().manual_seed(2718)
+    one = torch.tensor(1.0)
+    problems, wants = [], []
+    for case in range(14):
+        M = int(torch.randint(129, 1400, (1,), generator=rng))
+        N = int(torch.randint(129, 1400, (1,), generator=rng))
+        K = 16 * int(torch.randint(16, 130, (1,), generator=rng))
+        fa, fb = (O.E5M2, O.E4M3) if case % 3 else (O.E4M3, O.E4M3)
+        a = torch.randint(-4, 5, (M, K), generator=rng).float()
+        b = torch.randint(-4, 5, (N, K), generator=rng).float()
+        A, B = from_bytes(O.cast_to_fp8(a, one, fa), 1.0, fa), from_bytes(O.cast_to_fp8(b, one, fb), 1.0, fb)
+        want = a @ b.t()
+        od = (torch.float32, torch.bfloat16, torch.float16)[case % 3]
+        assert torch.equal(gpu_gemm_nt(A, B, od).cpu(), want.to(od)), (M, N, K, od)
+        problems.append((A, B, od, None))
+        wants.append(want.to(od))
+    for got, want in zip(_gemm_nt_batch(problems), wants):
+        assert torch.equal(got.cpu(), want)
