@@ -127,30 +127,30 @@ def _quantize(cls, tensor: torch.Tensor, dtype: DTypes, state: Optional[DelayedS
         out_t = torch.empty((cols, rows), dtype=torch.uint8, device=dev)
     scalars = torch.empty(2, dtype=torch.float32, device=dev)  # [amax, scale used]
     amax, scale = scalars[0], scalars[1]
-    ws = nt.workspace(dev)
-    st = nt.stream_ptr(dev)
+    ws, st = nt.workspace_and_stream(dev)
     fmt = _FMT[dtype]
     xd = nt.TORCH_TO_NT[x.dtype]
+    amax_p = scalars.data_ptr()
+    scale_p = amax_p + 4
     if state is None:
-        nt.check(nt.lib.ntfp8_quantize_current(x.data_ptr(), xd, rows, cols, fmt, _int_margin(margin), amax.data_ptr(),
-                                               scale.data_ptr(), out.data_ptr(), nt.ptr(out_t), None, 0, None,
+        nt.check(nt.lib.ntfp8_quantize_current(x.data_ptr(), xd, rows, cols, fmt, _int_margin(margin), amax_p,
+                                               scale_p, out.data_ptr(), nt.ptr(out_t), None, 0, None,
                                                ws.data_ptr(), st), "ntfp8_quantize_current")
     else:
         assert state.dtype == dtype, "delayed-scaling state was created for another format"
         assert state._buf.device == dev
+        state_p = state._buf.data_ptr()   # [scale, hist[0..H-1]]
         if not state.initialised:
-            nt.check(nt.lib.ntfp8_quantize_current(x.data_ptr(), xd, rows, cols, fmt, state.margin, amax.data_ptr(),
-                                                   scale.data_ptr(), out.data_ptr(), nt.ptr(out_t),
-                                                   state.amax_history.data_ptr(), state.history_len,
-                                                   state.scale.data_ptr(), ws.data_ptr(), st),
+            nt.check(nt.lib.ntfp8_quantize_current(x.data_ptr(), xd, rows, cols, fmt, state.margin, amax_p,
+                                                   scale_p, out.data_ptr(), nt.ptr(out_t),
+                                                   state_p + 4, state.history_len, state_p, ws.data_ptr(), st),
                      "ntfp8_quantize_current")
             # only while the role has never seen a usable amax: one host read to learn whether it has now
             a = float(amax.item())
             state.initialised = a > 0.0 and a != float("inf")
         else:
             nt.check(nt.lib.ntfp8_quantize_delayed(x.data_ptr(), xd, rows, cols, fmt, state.margin,
-                                                   state.scale.data_ptr(), state.amax_history.data_ptr(),
-                                                   state.history_len, amax.data_ptr(), scale.data_ptr(),
+                                                   state_p, state_p + 4, state.history_len, amax_p, scale_p,
                                                    out.data_ptr(), nt.ptr(out_t), ws.data_ptr(), st),
                      "ntfp8_quantize_delayed")
     meta = FP8Meta(amax, scale, dtype)
