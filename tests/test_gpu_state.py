@@ -117,3 +117,72 @@ def test_optimizer_hook_requantises_after_every_step():
     before = model[0].weight.data.as_subclass(torch.Tensor).clone()
     opt.step()
     assert torch.equal(model[0].weight.data.as_subclass(torch.Tensor), before)  # detached: no refresh any more
+
+
+def test_step_replayed_as_a_graph_matches_eager():
+    """The library allocates nothing, synchronises nothing and leaves its reduction workspace zero, so a
+    training step can be captured once and replayed: three replays with fresh inputs, with eager work and
+    synchronisations in between, against an eager twin that starts from the same state."""
+    import copy
+
+    from nanotron_amd.fp8 import FP8Linear
+    from nanotron_amd.fp8.optim import requantize_fp8_weights
+
+    def build():
+        torch.manual_seed(11)
+        return nn.Sequential(FP8Linear(256, 512, bias=False, device="cuda", delayed_scaling=True, out_dtype=torch.bfloat16),
+                             FP8Linear(512, 256, bias=False, device="cuda", delayed_scaling=True, out_dtype=torch.bfloat16))
+
+    def inputs(i):
+        return (O.normal_tensor(300 + i, (384, 256), 1.0 + 0.1 * i, torch.bfloat16).cuda(),
+                O.normal_tensor(400 + i, (384, 256), 1e-3, torch.bfloat16).cuda())
+
+    def step(model, x, gy):
+        requantize_fp8_weights(model)
+        x.grad = None
+        y = model(x)
+        y.backward(gy)
+        return y
+
+    g_model, e_model = build(), build()
+    sx = torch.zeros(384, 256, dtype=torch.bfloat16, device="cuda", requires_grad=True)
+    sgy = torch.zeros(384, 256, dtype=torch.bfloat16, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):   # warm-up on the capture stream: every scaling state has seen an amax
+        for i in range(2):
+            x, gy = inputs(i)
+            with torch.no_grad():
+                sx.copy_(x)
+                sgy.copy_(gy)
+            step(g_model, sx, sgy)
+    torch.cuda.current_stream().wait_stream(side)
+    for i in range(2):
+        x, gy = inputs(i)
+        step(e_model, x.requires_grad_(True), gy)
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    x, gy = inputs(2)
+    with torch.no_grad():
+        sx.copy_(x)
+        sgy.copy_(gy)
+    with torch.cuda.graph(graph):
+        sy = step(g_model, sx, sgy)
+    # capture does not execute: bring the eager twin to the same point by not stepping it either
+    for i in range(2, 5):
+        x, gy = inputs(i)
+        with torch.no_grad():
+            sx.copy_(x)
+            sgy.copy_(gy)
+        graph.replay()
+        xe = x.clone().requires_grad_(True)
+        ye = step(e_model, xe, gy)
+        _ = (ye.float() @ ye.float().t()).sum().item()   # unrelated eager work and a synchronisation in between
+        assert torch.equal(sy, ye)
+        assert torch.equal(sx.grad, xe.grad)
+        for lg, le in zip(g_model, e_model):
+            assert torch.equal(lg.weight.main_grad if lg.weight.dtype != torch.float32 else lg.weight.grad,
+                               le.weight.main_grad if le.weight.dtype != torch.float32 else le.weight.grad)
+            for role in lg.scaling:
+                assert torch.equal(lg.scaling[role]._buf, le.scaling[role]._buf)
