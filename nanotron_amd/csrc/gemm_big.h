@@ -172,8 +172,11 @@ struct BigLaunch {
 template <int FA, int FB, int MI>
 __global__ __launch_bounds__(MI == 8 ? kBigThreads : 2 * kBigThreads)
 void gemm_nt_big_kernel(const BigLaunch L) {
-    __shared__ __attribute__((aligned(1024))) uint8_t sA[2][32 * MI * kBK];
-    __shared__ __attribute__((aligned(1024))) uint8_t sB[2][kBigN * kBK];
+    // whole tiles: 2 stages of 64 KB; half tiles: 3 stages of 48 KB (their loads go straight to LDS and need the
+    // extra stage to have two K-tiles of flight time, see below)
+    constexpr int NS = MI == 8 ? 2 : 3;
+    __shared__ __attribute__((aligned(1024))) uint8_t sA[NS][32 * MI * kBK];
+    __shared__ __attribute__((aligned(1024))) uint8_t sB[NS][kBigN * kBK];
 
     // ---- which tile (or half tile) of which problem is this workgroup's ----------------------------
     int pid = blockIdx.x;
@@ -252,8 +255,9 @@ void gemm_nt_big_kernel(const BigLaunch L) {
 #pragma unroll
             for (int j = 0; j < kBigNJ; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-        // load number `l` (0 .. NL-1, A loads first) of K-tile `ktile` into stage `s`
-        auto issue = [&](int s, int ktile, int l) {
+        // load number `l` (0 .. NL-1, A loads first) of K-tile `ktile` straight into its LDS stage, ktile mod NS
+        auto issue = [&](int ktile, int l) {
+            const int s = ktile % NS;
             if (l < LA)
                 lds_load16(ra, (lds_ptr)(uintptr_t)&sA[s][(wave + kBigWaves * l) * 1024], a_off[l], ktile * kBK);
             else
@@ -287,14 +291,15 @@ void gemm_nt_big_kernel(const BigLaunch L) {
 
         v4i fa[MI][2], fb[4][2];
 
-        // A K-tile kt lives in LDS stage kt & 1 and is computed in two parts:
+        // A K-tile kt lives in LDS stage kt mod NS and is computed in two parts:
         //   front(kt): MFMA groups 0-5.  Entered with fa[] = the tile's A fragments and fb[0], fb[1] = its first
-        //              two B fragments; streams B fragments 2..7; queues the loads of tile kt + 1 that are not
-        //              yet queued; ends with the barrier that publishes tile kt + 1 and releases stage kt & 1.
-        //   back(kt):  MFMA groups 6-7, interleaved per A fragment; refills fa[] / fb[0], fb[1] from tile kt + 1
-        //              and queues the first kBackLoads loads of tile kt + 2 into the released stage.
+        //              two B fragments; streams B fragments 2..7; ends with the barrier that publishes tile
+        //              kt + 1 and releases the stage of tile kt.
+        //   back(kt):  MFMA groups 6-7, interleaved per A fragment; refills fa[] / fb[0], fb[1] from tile kt + 1.
         // The K loop runs back(kt); front(kt + 1), so that its back edge sits right behind the barrier, where no
-        // LDS read is outstanding.
+        // LDS read is outstanding.  With direct-to-LDS loads (half tiles) the stage released by the barrier of
+        // tile kt is refilled with tile kt + NS between that barrier and the next: half of the loads under
+        // back(kt), the rest under groups 0-1 of front(kt + 1).
         //
         // An MFMA occupies the matrix pipe for 32 cycles and the wave issues in order, so whatever stands between
         // two MFMAs must issue within that time or the pipe idles.  The code below therefore puts at most one
@@ -302,59 +307,61 @@ void gemm_nt_big_kernel(const BigLaunch L) {
         // pair keeps the compiler from regrouping them.
         constexpr int kBackLoads = NL / 2;
         constexpr int kFrontLoads = NL - kBackLoads;   // half under group 0, half under group 1
-        auto front = [&](auto loads_tag, auto barrier_tag, int kt) {
-            constexpr bool loads = decltype(loads_tag)::value, barrier = decltype(barrier_tag)::value;
-            const int s = kt & 1;
+        // loads: queue the second half of tile kt + NS - 1; WAIT (>= 0): barrier, after all but the newest WAIT
+        // loads of this wave have landed (-1: no barrier)
+        auto front = [&](auto loads_tag, auto wait_tag, int kt) {
+            constexpr bool loads = decltype(loads_tag)::value;
+            constexpr int WAIT = decltype(wait_tag)::value;
+            const int s = kt % NS;
             sched_fence();
 #pragma unroll
             for (int j = 0; j < 6; ++j) {
-                int l = kBackLoads + j * (kFrontLoads / 2);           // next load of tile kt + 1 to queue
+                int l = kBackLoads + j * (kFrontLoads / 2);           // next load to queue
                 const int lend = (loads && j < 2) ? l + kFrontLoads / 2 : l;
 #pragma unroll
                 for (int i = 0; i < MI; ++i) {
                     acc[i][j] = mfma_16x16x128<FA, FB>(frag(fb[j & 3]), frag(fa[i]), acc[i][j]);
                     if (i == 0) fb[(j + 2) & 3][0] = rd_b(s, j + 2, 0);
                     else if (i == 2) fb[(j + 2) & 3][1] = rd_b(s, j + 2, 1);
-                    else if (l < lend) issue(s ^ 1, kt + 1, l++);
+                    else if (l < lend) issue(kt + NS - 1, l++);
                     if (i == MI - 1) {   // whatever did not get a slot of its own
-                        for (; l < lend; ++l) issue(s ^ 1, kt + 1, l);
+                        for (; l < lend; ++l) issue(kt + NS - 1, l);
                     }
                     sched_fence();
                 }
             }
-            if constexpr (barrier) {
-                // Every fragment of tile kt is in registers (or in flight): after the barrier stage s may be
-                // overwritten, and tile kt + 1 is complete in stage s ^ 1.
+            if constexpr (WAIT >= 0) {
+                // Every fragment of tile kt is in registers (or in flight): after the barrier its stage may be
+                // overwritten, and tile kt + 1 is complete in the next stage.
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(WAIT) : "memory");
                 wg_barrier();
             }
         };
         auto back = [&](auto loads_tag, auto prefetch_tag, int kt) {
             constexpr bool loads = decltype(loads_tag)::value, prefetch = decltype(prefetch_tag)::value;
-            const int s = kt & 1;
-            if (loads && kt + 3 == KT) poison_tail();   // the loads queued below are the first of the last tile
+            const int s1 = (kt + 1) % NS;
             sched_fence();
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
                 // fa[i] is dead after its two MFMAs; it is refilled with the fragment of the next tile one step later
                 acc[i][6] = mfma_16x16x128<FA, FB>(frag(fb[2]), frag(fa[i]), acc[i][6]);
                 if (prefetch && i > 0) {
-                    fa[i - 1][0] = rd_a(s ^ 1, i - 1, 0);
-                    fa[i - 1][1] = rd_a(s ^ 1, i - 1, 1);
+                    fa[i - 1][0] = rd_a(s1, i - 1, 0);
+                    fa[i - 1][1] = rd_a(s1, i - 1, 1);
                 }
                 sched_fence();
                 acc[i][7] = mfma_16x16x128<FA, FB>(frag(fb[3]), frag(fa[i]), acc[i][7]);
                 if constexpr (loads) {   // loads [i kBackLoads / MI, (i + 1) kBackLoads / MI) ride on this step
 #pragma unroll
-                    for (int l = i * kBackLoads / MI; l < (i + 1) * kBackLoads / MI; ++l) issue(s, kt + 2, l);
+                    for (int l = i * kBackLoads / MI; l < (i + 1) * kBackLoads / MI; ++l) issue(kt + NS, l);
                 }
-                if (prefetch && i < 4) fb[i >> 1][i & 1] = rd_b(s ^ 1, i >> 1, i & 1);
+                if (prefetch && i < 4) fb[i >> 1][i & 1] = rd_b(s1, i >> 1, i & 1);
                 sched_fence();
             }
             if constexpr (prefetch) {
-                fa[MI - 1][0] = rd_a(s ^ 1, MI - 1, 0);
-                fa[MI - 1][1] = rd_a(s ^ 1, MI - 1, 1);
+                fa[MI - 1][0] = rd_a(s1, MI - 1, 0);
+                fa[MI - 1][1] = rd_a(s1, MI - 1, 1);
             }
             sched_fence();
         };
@@ -413,10 +420,10 @@ void gemm_nt_big_kernel(const BigLaunch L) {
             };
             // prologue: tiles 0 and 1 straight into LDS
 #pragma unroll
-            for (int l = 0; l < NL; ++l) issue(0, 0, l);
+            for (int l = 0; l < NL; ++l) issue(0, l);
             if (KT == 2) poison_tail();
 #pragma unroll
-            for (int l = 0; l < NL; ++l) issue(1, 1, l);
+            for (int l = 0; l < NL; ++l) issue(1, l);
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");   // tile 0 has landed, tile 1 may still be in flight
             wg_barrier();
 #pragma unroll
@@ -452,13 +459,26 @@ void gemm_nt_big_kernel(const BigLaunch L) {
             back(No{}, No{}, f);
         } else {
         // ---- half tiles: loads go straight into LDS (the register budget has no room for staging) --------
-        // prologue: tile 0 completely, the first kBackLoads loads of tile 1
+        // Three stages: the loads of tile t are queued while tile t - 3's stage is the one just released, i.e.
+        // two K-tiles before tile t is published.  A half-tile K-tile is only 32 MFMAs (about 0.55 us): with
+        // two stages the loads had half a K-tile to arrive, less than an L2 hit takes.
+        using Wait = std::integral_constant<int, NL>;   // the NL loads of the newest tile may still be in flight
+        using WaitAll = std::integral_constant<int, 0>;
+        using NoBarrier = std::integral_constant<int, -1>;
+        // prologue: tiles 0, 1 and (if there is one) 2
 #pragma unroll
-        for (int l = 0; l < NL; ++l) issue(0, 0, l);
+        for (int l = 0; l < NL; ++l) issue(0, l);
         if (KT == 2) poison_tail();
 #pragma unroll
-        for (int l = 0; l < kBackLoads; ++l) issue(1, 1, l);
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBackLoads) : "memory");
+        for (int l = 0; l < NL; ++l) issue(1, l);
+        if (KT > 2) {
+            if (KT == 3) poison_tail();
+#pragma unroll
+            for (int l = 0; l < NL; ++l) issue(2, l);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NL) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
+        }
         wg_barrier();
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
@@ -468,15 +488,23 @@ void gemm_nt_big_kernel(const BigLaunch L) {
 #pragma unroll
         for (int h = 0; h < 4; ++h) fb[h >> 1][h & 1] = rd_b(0, h >> 1, h & 1);
 
-        front(Yes{}, Yes{}, 0);
-        int kt = 0;
-        for (; kt < KT - 2; ++kt) {
-            back(Yes{}, Yes{}, kt);
-            front(Yes{}, Yes{}, kt + 1);
+        // front(0) queues nothing (tile 3 goes into the stage that front(0) itself still reads)
+        if (KT > 2) front(No{}, Wait{}, 0);
+        else front(No{}, WaitAll{}, 0);
+        int f = 1;
+        for (; f + 2 < KT; ++f) {   // tile f + 2 is loaded during back(f - 1); front(f)
+            if (f + 3 == KT) poison_tail();
+            back(Yes{}, Yes{}, f - 1);
+            front(Yes{}, Wait{}, f);
         }
-        back(No{}, Yes{}, kt);        // kt = KT - 2: nothing left to load
-        front(No{}, No{}, kt + 1);
-        back(No{}, No{}, kt + 1);
+        if (f + 1 < KT) {   // f = KT - 2 >= 1: nothing left to load
+            back(No{}, Yes{}, f - 1);
+            front(No{}, WaitAll{}, f);
+            ++f;
+        }
+        back(No{}, Yes{}, f - 1);   // f = KT - 1
+        front(No{}, NoBarrier{}, f);
+        back(No{}, No{}, f);
         }
 
         // output type and accumulation are properties of the problem, not of the kernel
