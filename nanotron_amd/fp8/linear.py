@@ -24,16 +24,18 @@ class FP8Linear(nn.Linear):
     """nn.Linear whose matmuls run in FP8 (reference: src/nanotron/fp8/linear.py:24-66).
 
     Positional signature as the reference.  Keyword-only extensions, all defaulting to the
-    reference's behaviour: `out_dtype` (None = fp32 output, kernel.py:24,28), `delayed_scaling`
+    reference's behaviour: `dtype` (of the master weight and bias, as nn.Linear's), `out_dtype`
+    (None = fp32 output, kernel.py:24,28), `delayed_scaling`
     (False = scale every tensor from its own amax), `amax_history_len`, `margin`,
     `accumulate_grad` (False = `weight.grad` is overwritten each backward, linear.py:110; True =
     the wgrad GEMM adds into the existing fp32 gradient in its epilogue).  With a bf16 / fp16
     master weight the fp32 weight gradient is stored as `weight.main_grad` instead of `.grad`."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, device: Optional[torch.device] = None,
-                 *, out_dtype: Optional[torch.dtype] = None, delayed_scaling: bool = False,
-                 amax_history_len: int = 16, margin: int = 0, accumulate_grad: bool = False):
-        super().__init__(in_features, out_features, bias, device)
+                 *, dtype: Optional[torch.dtype] = None, out_dtype: Optional[torch.dtype] = None,
+                 delayed_scaling: bool = False, amax_history_len: int = 16, margin: int = 0,
+                 accumulate_grad: bool = False):
+        super().__init__(in_features, out_features, bias, device, dtype)
         self.out_dtype = out_dtype
         self.accumulate_grad = accumulate_grad
         self.scaling = None
