@@ -125,9 +125,30 @@ typedef struct ntfp8_gemm_desc {
     void* D;
     int64_t M, N, K;
     int fmt_a, fmt_b, d_dtype, accumulate;
+    /* fp8 outputs only (d_dtype NTFP8_OUT_E4M3 / NTFP8_OUT_E5M2, below); ignored otherwise */
+    const float* scale_d;   /* device scalar: the result is multiplied by it before the cast */
+    void* D_t;              /* NULL, or [N, M] bytes: the transposed copy of D */
+    void* amax_workspace;   /* NULL, or NTFP8_WORKSPACE_BYTES, all zero: collects max|result| */
 } ntfp8_gemm_desc;
 #define NTFP8_MAX_BATCH 64
 int ntfp8_gemm_batch(const ntfp8_gemm_desc* problems, int count, void* stream);
+
+/* fp8 GEMM output ("return an fp8 tensor as output", the TODO at src/nanotron/fp8/linear.py:63-64):
+ * with d_dtype one of the two codes below, a problem of ntfp8_gemm_batch writes
+ *   D[m,n] = sat_rne_fp8(r * *scale_d),  r = fp32 result as d_dtype NTFP8_F32 would store it,
+ * i.e. the bytes ntfp8_cast_to_fp8 makes of the fp32 output, NaN -> sign|0x7F included, and the same
+ * bytes transposed into D_t if given.  accumulate must be 0.  The amax of r cannot be known before
+ * the GEMM has run, so the scale is one decided earlier (delayed scaling); the GEMM leaves max|r| in
+ * amax_workspace, and ntfp8_amax_finalize, queued behind it on the same stream, turns that into the
+ * bookkeeping of ntfp8_quantize_delayed:
+ *   *amax_out = max|r| (NaN if any r is); hist <- roll(hist), hist[0] = amax;
+ *   *scale_used_out = old *scale_state; *scale_state = update_scaling_factor(max(hist), old);
+ * and zeroes the workspace again.  scale_d usually is scale_state.  amax_history may be NULL
+ * (history_len 0): then only *amax_out and *scale_used_out are written. */
+#define NTFP8_OUT_E4M3 3
+#define NTFP8_OUT_E5M2 4
+int ntfp8_amax_finalize(void* workspace, int fmt, int margin, float* scale_state, float* amax_history,
+                        int history_len, float* amax_out, float* scale_used_out, void* stream);
 
 #ifdef __cplusplus
 }

@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libntfp8.so")
 
 E4M3, E5M2 = 0, 1
 F32, F16, BF16 = 0, 1, 2
+OUT_E4M3, OUT_E5M2 = 3, 4  # d_dtype of an fp8 GEMM output
 WORKSPACE_BYTES = 2048
 
 TORCH_TO_NT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
@@ -35,7 +36,8 @@ class GemmDesc(ctypes.Structure):
     """`ntfp8_gemm_desc` of include/ntfp8.h."""
     _fields_ = [("A", _vp), ("scale_a", _vp), ("B", _vp), ("scale_b", _vp), ("D", _vp),
                 ("M", _i64), ("N", _i64), ("K", _i64),
-                ("fmt_a", _i), ("fmt_b", _i), ("d_dtype", _i), ("accumulate", _i)]
+                ("fmt_a", _i), ("fmt_b", _i), ("d_dtype", _i), ("accumulate", _i),
+                ("scale_d", _vp), ("D_t", _vp), ("amax_workspace", _vp)]
 
 
 SIGNATURES = {
@@ -51,6 +53,7 @@ SIGNATURES = {
     "ntfp8_transpose": (_i, [_vp, _i64, _i64, _vp, _vp]),
     "ntfp8_gemm": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i64, _i64, _i64, _i, _vp]),
     "ntfp8_gemm_batch": (_i, [_c.POINTER(GemmDesc), _i, _vp]),
+    "ntfp8_amax_finalize": (_i, [_vp, _i, _i, _vp, _vp, _i, _vp, _vp, _vp]),
 }
 
 for _name, (_res, _args) in SIGNATURES.items():

@@ -10,6 +10,7 @@ int run_dequant(const void* in, int fmt, const float* scale, int64_t n, void* ou
 int run_transpose(const void* in, int64_t rows, int64_t cols, void* out, hipStream_t st);
 int run_update_scale(const float* amax, const float* old_scale, int fmt, int margin, float* out, int64_t n,
                      hipStream_t st);
+int run_amax_finalize(Workspace* ws, const ScalarIO& io, hipStream_t st);
 int run_gemm(const GemmDesc& g, hipStream_t st);
 int run_gemm_batch(const GemmDesc* g, int n, hipStream_t st);
 
@@ -20,7 +21,7 @@ constexpr int kMaxMargin = 126;
 
 bool fmt_ok(int f) { return f == NTFP8_E4M3 || f == NTFP8_E5M2; }
 bool dtype_ok(int d) { return d == NTFP8_F32 || d == NTFP8_F16 || d == NTFP8_BF16; }
-size_t dtype_size(int d) { return d == NTFP8_F32 ? 4 : 2; }
+size_t dtype_size(int d) { return d == NTFP8_F32 ? 4 : (is_fp8_out(d) ? 1 : 2); }
 bool is_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 // rows * cols as a positive int64, or false
@@ -58,7 +59,9 @@ int check_outputs(const void* x, int x_dtype, int64_t n, const void* out, const 
 // argument checks of one GEMM problem; fills the launchers' descriptor
 int check_gemm(const ntfp8_gemm_desc& p, GemmDesc* g) {
     if (!p.A || !p.B || !p.D || !p.scale_a || !p.scale_b) return NTFP8_ERR_NULL;
-    if (!fmt_ok(p.fmt_a) || !fmt_ok(p.fmt_b) || !dtype_ok(p.d_dtype)) return NTFP8_ERR_ENUM;
+    const bool fp8_out = is_fp8_out(p.d_dtype);
+    if (!fmt_ok(p.fmt_a) || !fmt_ok(p.fmt_b) || !(dtype_ok(p.d_dtype) || fp8_out)) return NTFP8_ERR_ENUM;
+    if (fp8_out && !p.scale_d) return NTFP8_ERR_NULL;
     const int64_t M = p.M, N = p.N, K = p.K;
     if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffff00LL || N > 0x7fffff00LL || K > 0x7fffff00LL) return NTFP8_ERR_SIZE;
     int64_t mn, mk, nk;
@@ -69,7 +72,19 @@ int check_gemm(const ntfp8_gemm_desc& p, GemmDesc* g) {
         return NTFP8_ERR_ALIGN;
     const size_t db = (size_t)mn * dtype_size(p.d_dtype);
     if (overlap(p.A, (size_t)mk, p.D, db) || overlap(p.B, (size_t)nk, p.D, db)) return NTFP8_ERR_ALIAS;
-    *g = GemmDesc{p.A, p.fmt_a, p.scale_a, p.B, p.fmt_b, p.scale_b, p.D, p.d_dtype, (int)M, (int)N, (int)K, p.accumulate ? 1 : 0};
+    *g = GemmDesc{p.A, p.fmt_a, p.scale_a, p.B, p.fmt_b, p.scale_b, p.D, p.d_dtype, (int)M, (int)N, (int)K, p.accumulate ? 1 : 0,
+                  nullptr, nullptr, nullptr};
+    if (fp8_out) {
+        if (!is_aligned(p.scale_d, 4) || (p.amax_workspace && !is_aligned(p.amax_workspace, 4))) return NTFP8_ERR_ALIGN;
+        if (p.D_t && (overlap(p.A, (size_t)mk, p.D_t, db) || overlap(p.B, (size_t)nk, p.D_t, db) || overlap(p.D, db, p.D_t, db)))
+            return NTFP8_ERR_ALIAS;
+        if (p.amax_workspace &&
+            (overlap(p.amax_workspace, NTFP8_WORKSPACE_BYTES, p.D, db) || (p.D_t && overlap(p.amax_workspace, NTFP8_WORKSPACE_BYTES, p.D_t, db))))
+            return NTFP8_ERR_ALIAS;
+        g->sd = p.scale_d;
+        g->Dt = p.D_t;
+        g->ws = p.amax_workspace;
+    }
     return NTFP8_OK;
 }
 
@@ -201,7 +216,8 @@ int ntfp8_transpose(const void* in, int64_t rows, int64_t cols, void* out, void*
 
 int ntfp8_gemm(const void* A, int fmt_a, const float* scale_a, const void* B, int fmt_b, const float* scale_b, void* D,
                int d_dtype, int64_t M, int64_t N, int64_t K, int accumulate, void* stream) {
-    const ntfp8_gemm_desc p = {A, scale_a, B, scale_b, D, M, N, K, fmt_a, fmt_b, d_dtype, accumulate};
+    if (is_fp8_out(d_dtype)) return NTFP8_ERR_UNSUPPORTED;   // fp8 outputs carry more arguments: ntfp8_gemm_batch
+    const ntfp8_gemm_desc p = {A, scale_a, B, scale_b, D, M, N, K, fmt_a, fmt_b, d_dtype, accumulate, nullptr, nullptr, nullptr};
     GemmDesc g;
     const int rc = check_gemm(p, &g);
     if (rc) return rc;
@@ -216,18 +232,40 @@ int ntfp8_gemm_batch(const ntfp8_gemm_desc* problems, int count, void* stream) {
         const int rc = check_gemm(problems[i], &g[i]);
         if (rc) return rc;
     }
-    // independence: an output overlaps nothing of any other problem
+    // independence: an output (D, its transposed copy, its amax slots) overlaps nothing of any other problem
     for (int i = 0; i < count; ++i) {
         const size_t di = (size_t)g[i].M * g[i].N * dtype_size(g[i].d_dtype);
+        const void* outs_i[3] = {g[i].D, g[i].Dt, g[i].ws};
+        const size_t size_i[3] = {di, di, NTFP8_WORKSPACE_BYTES};
         for (int j = 0; j < count; ++j) {
             if (i == j) continue;
             const size_t dj = (size_t)g[j].M * g[j].N * dtype_size(g[j].d_dtype);
-            if (overlap(g[i].D, di, g[j].A, (size_t)g[j].M * g[j].K) || overlap(g[i].D, di, g[j].B, (size_t)g[j].N * g[j].K) ||
-                (i < j && overlap(g[i].D, di, g[j].D, dj)))
-                return NTFP8_ERR_ALIAS;
+            const void* outs_j[3] = {g[j].D, g[j].Dt, g[j].ws};
+            const size_t size_j[3] = {dj, dj, NTFP8_WORKSPACE_BYTES};
+            for (int a = 0; a < 3; ++a) {
+                if (!outs_i[a]) continue;
+                if (overlap(outs_i[a], size_i[a], g[j].A, (size_t)g[j].M * g[j].K) ||
+                    overlap(outs_i[a], size_i[a], g[j].B, (size_t)g[j].N * g[j].K))
+                    return NTFP8_ERR_ALIAS;
+                for (int b = 0; b < 3; ++b)
+                    if (i < j && outs_j[b] && overlap(outs_i[a], size_i[a], outs_j[b], size_j[b])) return NTFP8_ERR_ALIAS;
+            }
         }
     }
     return run_gemm_batch(g, count, static_cast<hipStream_t>(stream));
+}
+
+int ntfp8_amax_finalize(void* workspace, int fmt, int margin, float* scale_state, float* amax_history, int history_len,
+                        float* amax_out, float* scale_used_out, void* stream) {
+    if (!workspace || !scale_state || !amax_out) return NTFP8_ERR_NULL;
+    if (!fmt_ok(fmt)) return NTFP8_ERR_ENUM;
+    if (margin < -kMaxMargin || margin > kMaxMargin) return NTFP8_ERR_SIZE;
+    if (amax_history ? (history_len < 1 || history_len > kMaxHistory) : history_len != 0) return NTFP8_ERR_SIZE;
+    if (!is_aligned(workspace, 4) || !is_aligned(scale_state, 4) || !is_aligned(amax_out, 4) ||
+        (amax_history && !is_aligned(amax_history, 4)) || (scale_used_out && !is_aligned(scale_used_out, 4)))
+        return NTFP8_ERR_ALIGN;
+    ScalarIO io = {nullptr, amax_out, scale_used_out, scale_state, amax_history, history_len, fmt, margin};
+    return run_amax_finalize(static_cast<Workspace*>(workspace), io, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -139,7 +139,13 @@ struct GemmDesc {
     int d_dtype;
     int M, N, K;
     int accumulate;
+    // fp8 outputs (d_dtype NTFP8_OUT_*): scale applied before the cast, optional transposed copy, optional amax slots
+    const float* sd;
+    void* Dt;
+    void* ws;
 };
+
+__host__ __device__ inline bool is_fp8_out(int d_dtype) { return d_dtype == NTFP8_OUT_E4M3 || d_dtype == NTFP8_OUT_E5M2; }
 
 // compute units of the current device (cached per device)
 inline int cu_count() {

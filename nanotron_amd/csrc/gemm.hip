@@ -25,7 +25,7 @@ template <int FA, int FB, int DT, bool kAcc>
 __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                                void* __restrict__ Dv, const float* __restrict__ scale_a,
                                                                const float* __restrict__ scale_b, int M, int N, int K,
-                                                               int tiles_m, int tiles_n) {
+                                                               int tiles_m, int tiles_n, Fp8Out fp8) {
     __shared__ __attribute__((aligned(16))) uint8_t sA[kBM * kBK];
     __shared__ __attribute__((aligned(16))) uint8_t sB[kBN * kBK];
 
@@ -106,7 +106,15 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(const uint8_t* __
     }
 
     const float alpha = (1.0f / *scale_a) * (1.0f / *scale_b);
-    store_wave_tile<DT, kAcc, 2, 2>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
+    if constexpr (DT == NTFP8_OUT_E4M3 || DT == NTFP8_OUT_E5M2) {
+        constexpr int F = DT == NTFP8_OUT_E4M3 ? kE4M3 : kE5M2;
+        const float scale_d = *fp8.scale;
+        const uint32_t amax = store_wave_tile_fp8<F, 2, 2>(acc, static_cast<uint8_t*>(Dv), fp8.Dt, alpha, scale_d,
+                                                           scale_is_degenerate(scale_d), M, N, m0 + wm, n0 + wn, lane);
+        publish_amax(amax, fp8.ws);
+    } else {
+        store_wave_tile<DT, kAcc, 2, 2>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
+    }
 }
 
 // Any K / alignment: one output element per thread, table-free decode through the hardware
@@ -114,26 +122,39 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(const uint8_t* __
 template <int FA, int FB, int DT, bool kAcc>
 __global__ void gemm_nt_naive_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, void* __restrict__ Dv,
                                      const float* __restrict__ scale_a, const float* __restrict__ scale_b, int M, int N,
-                                     int K) {
+                                     int K, Fp8Out fp8) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (int64_t)M * N) return;
-    const int m = (int)(idx / N), n = (int)(idx % N);
+    const bool live = idx < (int64_t)M * N;
+    if (!live && !(DT == NTFP8_OUT_E4M3 || DT == NTFP8_OUT_E5M2)) return;
+    const int m = live ? (int)(idx / N) : 0, n = live ? (int)(idx % N) : 0;
     float acc = 0.0f;
-    for (int k = 0; k < K; ++k) {
+    for (int k = 0; live && k < K; ++k) {
         const float a = FA == kE4M3 ? __builtin_amdgcn_cvt_f32_fp8((int)A[(int64_t)m * K + k], 0)
                                     : __builtin_amdgcn_cvt_f32_bf8((int)A[(int64_t)m * K + k], 0);
         const float b = FB == kE4M3 ? __builtin_amdgcn_cvt_f32_fp8((int)B[(int64_t)n * K + k], 0)
                                     : __builtin_amdgcn_cvt_f32_bf8((int)B[(int64_t)n * K + k], 0);
         acc += a * b;
     }
-    typedef typename OutT<DT>::type O;
-    O* D = static_cast<O*>(Dv);
     float v = acc * ((1.0f / *scale_a) * (1.0f / *scale_b));
-    if constexpr (DT == NTFP8_F32) {
-        if constexpr (kAcc) v = v + D[idx];
-        D[idx] = v;
+    if constexpr (DT == NTFP8_OUT_E4M3 || DT == NTFP8_OUT_E5M2) {
+        // whole waves get here (the amax reduction runs over all 64 lanes); lanes past the end hold zeros
+        constexpr int F = DT == NTFP8_OUT_E4M3 ? kE4M3 : kE5M2;
+        uint32_t amax = 0;
+        const uint32_t w = quant4<F>(v, 0.0f, 0.0f, 0.0f, *fp8.scale, true, amax);
+        if (live) {
+            static_cast<uint8_t*>(Dv)[idx] = (uint8_t)w;
+            if (fp8.Dt) fp8.Dt[(int64_t)n * M + m] = (uint8_t)w;
+        }
+        publish_amax(amax, fp8.ws);
     } else {
-        D[idx] = OutT<DT>::cvt(v);
+        typedef typename OutT<DT>::type O;
+        O* D = static_cast<O*>(Dv);
+        if constexpr (DT == NTFP8_F32) {
+            if constexpr (kAcc) v = v + D[idx];
+            D[idx] = v;
+        } else {
+            D[idx] = OutT<DT>::cvt(v);
+        }
     }
 }
 
@@ -149,13 +170,17 @@ static int path_of(const GemmDesc& g) {
     // the big kernel addresses its operands with 32-bit buffer offsets and wants enough tiles to matter
     const bool fits32 = (int64_t)(g.M + 256) * g.K < (1LL << 31) && (int64_t)(g.N + kBigN) * g.K < (1LL << 31);
     const bool worth = g.M > kBM && g.N > kBN && g.K >= 2 * kBK;
-    return (fits32 && worth) ? kPathBig : kPathSmall;
+    // its fp8 epilogue stores whole words through 32-bit buffer offsets
+    const bool fp8_ok = !is_fp8_out(g.d_dtype) ||
+                        (g.N % 16 == 0 && g.M % 4 == 0 && (int64_t)g.M * g.N < (1LL << 32) - 16 &&
+                         (reinterpret_cast<uintptr_t>(g.Dt) & 15) == 0);
+    return (fits32 && worth && fp8_ok) ? kPathBig : kPathSmall;
 }
 
 // One launch (plus one for the half-tile tail) of the big kernel over up to kBigMaxProblems problems of the
 // same operand formats.  Tiles are listed problem by problem, longest K first: the long tiles start together and
 // the shorter ones fill the rounds behind them.
-template <int FA, int FB>
+template <int FA, int FB, bool kFp8Out>
 static int launch_big(const GemmDesc* const* g, int n, hipStream_t st) {
     int order[kBigMaxProblems];
     for (int i = 0; i < n; ++i) order[i] = i;
@@ -184,6 +209,7 @@ static int launch_big(const GemmDesc* const* g, int n, hipStream_t st) {
         p.tile_begin = tiles;
         p.d_dtype = d.d_dtype;
         p.accumulate = d.accumulate;
+        p.fp8 = Fp8Out{d.sd, static_cast<uint8_t*>(d.Dt), static_cast<Workspace*>(d.ws)};
         tiles += p.tiles_m * p.tiles_n;
     }
     const int rem = tiles % cu_count();
@@ -191,9 +217,9 @@ static int launch_big(const GemmDesc* const* g, int n, hipStream_t st) {
     L.full_blocks = tiles - L.tail_tiles;
     L.round_size = cu_count();
     if (L.full_blocks > 0)
-        hipLaunchKernelGGL((gemm_nt_big_kernel<FA, FB, 8>), dim3(L.full_blocks), dim3(kBigThreads), 0, st, L);
+        hipLaunchKernelGGL((gemm_nt_big_kernel<FA, FB, 8, kFp8Out>), dim3(L.full_blocks), dim3(kBigThreads), 0, st, L);
     if (L.tail_tiles > 0)
-        hipLaunchKernelGGL((gemm_nt_big_kernel<FA, FB, 4>), dim3(2 * L.tail_tiles), dim3(kBigThreads), 0, st, L);
+        hipLaunchKernelGGL((gemm_nt_big_kernel<FA, FB, 4, kFp8Out>), dim3(2 * L.tail_tiles), dim3(kBigThreads), 0, st, L);
     return hipGetLastError() == hipSuccess ? NTFP8_OK : NTFP8_ERR_LAUNCH;
 }
 
@@ -201,26 +227,30 @@ template <int FA, int FB, int DT, bool kAcc>
 static int launch_small(const GemmDesc& g, int path, hipStream_t st) {
     const uint8_t* a = static_cast<const uint8_t*>(g.A);
     const uint8_t* b = static_cast<const uint8_t*>(g.B);
+    const Fp8Out fp8 = {g.sd, static_cast<uint8_t*>(g.Dt), static_cast<Workspace*>(g.ws)};
     if (path == kPathSmall) {
         const int tm = (g.M + kBM - 1) / kBM, tn = (g.N + kBN - 1) / kBN;
         hipLaunchKernelGGL((gemm_nt_kernel<FA, FB, DT, kAcc>), dim3(tm * tn), dim3(kGemmThreads), 0, st, a, b, g.D, g.sa,
-                           g.sb, g.M, g.N, g.K, tm, tn);
+                           g.sb, g.M, g.N, g.K, tm, tn, fp8);
     } else {
         const int64_t blocks = ((int64_t)g.M * g.N + 255) / 256;
         hipLaunchKernelGGL((gemm_nt_naive_kernel<FA, FB, DT, kAcc>), dim3((int)blocks), dim3(256), 0, st, a, b, g.D, g.sa,
-                           g.sb, g.M, g.N, g.K);
+                           g.sb, g.M, g.N, g.K, fp8);
     }
     return hipGetLastError() == hipSuccess ? NTFP8_OK : NTFP8_ERR_LAUNCH;
 }
 
 template <int FA, int FB>
 static int dispatch_fmt(const GemmDesc* const* g, int n, int path, hipStream_t st) {
-    if (path == kPathBig) return launch_big<FA, FB>(g, n, st);
+    if (path == kPathBig)
+        return is_fp8_out(g[0]->d_dtype) ? launch_big<FA, FB, true>(g, n, st) : launch_big<FA, FB, false>(g, n, st);
     const GemmDesc& d = *g[0];   // the small kernels take one problem
     if (d.d_dtype == NTFP8_F32)
         return d.accumulate ? launch_small<FA, FB, NTFP8_F32, true>(d, path, st)
                             : launch_small<FA, FB, NTFP8_F32, false>(d, path, st);
     if (d.d_dtype == NTFP8_BF16) return launch_small<FA, FB, NTFP8_BF16, false>(d, path, st);
+    if (d.d_dtype == NTFP8_OUT_E4M3) return launch_small<FA, FB, NTFP8_OUT_E4M3, false>(d, path, st);
+    if (d.d_dtype == NTFP8_OUT_E5M2) return launch_small<FA, FB, NTFP8_OUT_E5M2, false>(d, path, st);
     return launch_small<FA, FB, NTFP8_F16, false>(d, path, st);
 }
 
@@ -249,7 +279,8 @@ int run_gemm_batch(const GemmDesc* g, int n, hipStream_t st) {
         done[i] = true;
         if (path == kPathBig) {
             for (int j = i + 1; j < n && cnt < kBigMaxProblems; ++j)
-                if (!done[j] && g[j].fmt_a == g[i].fmt_a && g[j].fmt_b == g[i].fmt_b && path_of(g[j]) == kPathBig) {
+                if (!done[j] && g[j].fmt_a == g[i].fmt_a && g[j].fmt_b == g[i].fmt_b && path_of(g[j]) == kPathBig &&
+                    is_fp8_out(g[j].d_dtype) == is_fp8_out(g[i].d_dtype)) {
                     group[cnt++] = &g[j];
                     done[j] = true;
                 }

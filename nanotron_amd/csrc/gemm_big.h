@@ -136,6 +136,68 @@ __device__ __forceinline__ void store_wave_tile16(const v4f (&acc)[MI][NJ], void
     }
 }
 
+// 16 / 4 bytes per lane to global memory through a buffer descriptor; offsets past its size are dropped
+__device__ __forceinline__ void reg_store16(__amdgpu_buffer_rsrc_t r, uint32_t voff, v4i data) {
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, data), r, voff, 0, 0);
+}
+__device__ __forceinline__ void reg_store4(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t data) {
+    __builtin_amdgcn_raw_buffer_store_b32(data, r, voff, 0, 0);
+}
+
+// fp8 epilogue of one wave (layout as store_wave_tile16); returns the lane's max|r| as a bit pattern.
+// Shapes: N a multiple of 16, M a multiple of 4, M N < 2^32 (the launcher sends other shapes to the small kernel).
+// A lane's 4 consecutive n of a block are one word of D.  Row-major bytes: a 4 x 4 exchange of words between the
+// four lane rows and four neighbouring blocks gives lane row q the 16 consecutive n of block j0 + q, one 16-byte
+// store per lane and 64 contiguous bytes per output row and instruction.  Transposed bytes: a 4 x 4 byte transpose
+// inside each quad of lanes (4 consecutive m) turns the word into 4 consecutive m of one n.
+// All stores go through buffer descriptors of M N bytes: rows past the end fall outside and are dropped, columns
+// past the end get an offset that does; nothing is predicated, which keeps the scalar registers of the epilogue
+// (and with them the register budget of the K loop before it) small.
+template <int F, int MI, int NJ>
+__device__ __forceinline__ uint32_t store_wave_tile16_fp8(const v4f (&acc)[MI][NJ], uint8_t* __restrict__ D,
+                                                          uint8_t* __restrict__ Dt, float alpha, float scale_d, bool slow,
+                                                          int M, int N, int m_base, int n_base, int lane) {
+    static_assert(NJ % 4 == 0, "blocks are exchanged four at a time");
+    const int mrow = lane & 15, q = lane >> 4;
+    uint32_t amax = 0;
+    const uint32_t bytes = (uint32_t)M * (uint32_t)N;
+    const __amdgpu_buffer_rsrc_t rd = make_rsrc(D, bytes);
+    const __amdgpu_buffer_rsrc_t rt = make_rsrc(Dt, Dt ? bytes : 0u);
+    constexpr uint32_t kDropped = 0xfffffff0u;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+        const int m = m_base + i * 16 + mrow;
+        const int mq = m & ~3;
+        uint32_t w[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+            w[j] = quant4<F>(acc[i][j][0] * alpha, acc[i][j][1] * alpha, acc[i][j][2] * alpha, acc[i][j][3] * alpha, scale_d,
+                             slow, amax);
+        if (Dt) {   // uniform
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const uint32_t t = quad_transpose_bytes(w[j], lane);
+                const int nt = n_base + j * 16 + q * 4 + (lane & 3);
+                // nt >= N lies past the end of the [N, M] bytes by itself
+                reg_store4(rt, mq < M ? (uint32_t)nt * (uint32_t)M + (uint32_t)mq : kDropped, t);
+            }
+        }
+#pragma unroll
+        for (int j0 = 0; j0 < NJ; j0 += 4) {
+            uint32_t x0 = w[j0], x1 = w[j0 + 1], x2 = w[j0 + 2], x3 = w[j0 + 3];
+            swap_rows16(x0, x1);   // lane rows 1, 3 of a word <-> rows 0, 2 of the next block's word
+            swap_rows16(x2, x3);
+            swap_halves(x0, x2);   // lane rows 2, 3 <-> rows 0, 1 two blocks further on
+            swap_halves(x1, x3);
+            // lane row q now holds n 0-3, 4-7, 8-11, 12-15 of block j0 + q; m >= M lies past the end by itself
+            const int n = n_base + (j0 + q) * 16;
+            reg_store16(rd, n < N ? (uint32_t)m * (uint32_t)N + (uint32_t)n : kDropped, (v4i){(int)x0, (int)x1, (int)x2, (int)x3});
+        }
+    }
+    return amax;
+}
+
 // Launch geometry, computed on the host.  The first `full_blocks` tiles (in grouped order) are computed
 // whole by the MI = 8 kernel.  If the tile count leaves a partial last round over the CUs, the
 // remaining `tail_tiles` tiles are cut into two 128-row halves and computed by a second launch of
@@ -153,8 +215,9 @@ struct BigProblem {
     int M, N, K;
     int tiles_m, tiles_n;   // 256 x 256 tiles
     int tile_begin;         // position of this problem's first tile in the launch's tile list
-    int d_dtype;            // NTFP8_F32 / NTFP8_F16 / NTFP8_BF16
+    int d_dtype;            // NTFP8_F32 / NTFP8_F16 / NTFP8_BF16 / NTFP8_OUT_E4M3 / NTFP8_OUT_E5M2
     int accumulate;         // fp32 outputs only: D += result
+    Fp8Out fp8;             // fp8 outputs only
 };
 constexpr int kBigMaxProblems = 4;
 struct BigLaunch {
@@ -169,7 +232,9 @@ struct BigLaunch {
 // MI = 4 variant is held to half of it by declaring a launch bound of twice its real workgroup
 // size: given more registers than it needs, the compiler keeps its accumulators in a second
 // register set and copies them back and forth inside the K loop.
-template <int FA, int FB, int MI>
+// kFp8Out: every problem of the launch has an fp8 output (a kernel of its own: the other outputs' code stays as
+// the register allocator likes it).
+template <int FA, int FB, int MI, bool kFp8Out = false>
 __global__ __launch_bounds__(MI == 8 ? kBigThreads : 2 * kBigThreads)
 void gemm_nt_big_kernel(const BigLaunch L) {
     // whole tiles: 2 stages of 64 KB; half tiles: 3 stages of 48 KB (their loads go straight to LDS and need the
@@ -507,8 +572,18 @@ void gemm_nt_big_kernel(const BigLaunch L) {
         back(No{}, No{}, f);
         }
 
-        // output type and accumulation are properties of the problem, not of the kernel
-        if (P.d_dtype == NTFP8_BF16) {
+        // output type and accumulation are properties of the problem, not of the kernel (fp8 outputs apart)
+        if constexpr (kFp8Out) {
+            const float scale_d = *P.fp8.scale;
+            const bool slow = scale_is_degenerate(scale_d);
+            const uint32_t amax =
+                P.d_dtype == NTFP8_OUT_E4M3
+                    ? store_wave_tile16_fp8<kE4M3, MI, kBigNJ>(acc, static_cast<uint8_t*>(Dv), P.fp8.Dt, alpha, scale_d, slow, M,
+                                                               N, m0 + wm, n0 + wn, lane)
+                    : store_wave_tile16_fp8<kE5M2, MI, kBigNJ>(acc, static_cast<uint8_t*>(Dv), P.fp8.Dt, alpha, scale_d, slow, M,
+                                                               N, m0 + wm, n0 + wn, lane);
+            publish_amax(amax, P.fp8.ws);
+        } else if (P.d_dtype == NTFP8_BF16) {
             store_wave_tile16<NTFP8_BF16, false, MI, kBigNJ>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
         } else if (P.d_dtype == NTFP8_F16) {
             store_wave_tile16<NTFP8_F16, false, MI, kBigNJ>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);

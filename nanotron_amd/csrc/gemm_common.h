@@ -194,4 +194,104 @@ __device__ __forceinline__ void store_wave_tile(const v16f (&acc)[MI][NJ], void*
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// fp8 outputs: bytes = sat_rne_fp8(r * scale_d) of the descaled fp32 results r, optionally also
+// transposed, and max|r| for the delayed-scaling bookkeeping of the output.
+struct Fp8Out {
+    const float* scale;   // device scalar applied before the cast
+    uint8_t* Dt;          // NULL, or the [N, M] transposed copy
+    Workspace* ws;        // NULL, or the slots that collect max|r|
+};
+
+__device__ __forceinline__ bool scale_is_degenerate(float s) {   // 0, Inf or NaN: products can be NaN
+    const uint32_t b = __float_as_uint(s) & 0x7fffffffu;
+    return b == 0u || b >= kInfBits;
+}
+
+// Four results -> one word of fp8 bytes (first value in the low byte); amax_bits collects |r| as unsigned
+// bit patterns (NaN patterns compare above Inf).  The clamp turns a NaN into a number, so NaN bytes are patched
+// in afterwards; that is rare and sits behind a branch the whole wave takes or skips: `slow` (the scale is
+// degenerate, any product may be NaN) or some lane holding a NaN result.
+template <int F>
+__device__ __forceinline__ uint32_t quant4(float r0, float r1, float r2, float r3, float scale_d, bool slow,
+                                           uint32_t& amax_bits) {
+    const uint32_t a01 = max(__float_as_uint(r0) & 0x7fffffffu, __float_as_uint(r1) & 0x7fffffffu);
+    const uint32_t a23 = max(__float_as_uint(r2) & 0x7fffffffu, __float_as_uint(r3) & 0x7fffffffu);
+    const uint32_t a = max(a01, a23);
+    amax_bits = max(amax_bits, a);
+    const float y0 = r0 * scale_d, y1 = r1 * scale_d, y2 = r2 * scale_d, y3 = r3 * scale_d;
+    uint32_t w = cvt4<F>(sat<F>(y0), sat<F>(y1), sat<F>(y2), sat<F>(y3));
+    if (slow || __any(a > kInfBits)) {
+        w = patch_nan(w, 0, y0);
+        w = patch_nan(w, 1, y1);
+        w = patch_nan(w, 2, y2);
+        w = patch_nan(w, 3, y3);
+    }
+    return w;
+}
+
+// 4 x 4 byte transpose inside every quad of lanes: lane 4 a + k receives byte k of the words of lanes
+// 4 a .. 4 a + 3, in lane order from the low byte up.
+__device__ __forceinline__ uint32_t quad_transpose_bytes(uint32_t w, int lane) {
+    const uint32_t x0 = (uint32_t)__builtin_amdgcn_mov_dpp((int)w, 0x00, 0xf, 0xf, true);   // quad_perm [0,0,0,0]
+    const uint32_t x1 = (uint32_t)__builtin_amdgcn_mov_dpp((int)w, 0x55, 0xf, 0xf, true);   // [1,1,1,1]
+    const uint32_t x2 = (uint32_t)__builtin_amdgcn_mov_dpp((int)w, 0xaa, 0xf, 0xf, true);   // [2,2,2,2]
+    const uint32_t x3 = (uint32_t)__builtin_amdgcn_mov_dpp((int)w, 0xff, 0xf, 0xf, true);   // [3,3,3,3]
+    const uint32_t k = lane & 3;
+    const uint32_t sel = k | ((4u + k) << 8);   // V_PERM_B32: selector values 0-3 pick bytes of the second source, 4-7 of the first
+    const uint32_t t01 = __builtin_amdgcn_perm(x1, x0, sel);
+    const uint32_t t23 = __builtin_amdgcn_perm(x3, x2, sel);
+    return __builtin_amdgcn_perm(t23, t01, 0x05040100u);
+}
+
+// a word of 4 bytes to dst, whole if it may be (`vec`: dst + offsets are 4-byte aligned), else the bytes below `count`
+__device__ __forceinline__ void store_bytes4(uint8_t* dst, uint32_t w, bool vec, int count) {
+    if (vec && count >= 4) {
+        *reinterpret_cast<uint32_t*>(dst) = w;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (e < count) dst[e] = (uint8_t)(w >> (8 * e));
+    }
+}
+
+// one wave's share of max|r| into the launch's slots (slots of different workgroups sit on different lines)
+__device__ __forceinline__ void publish_amax(uint32_t lane_bits, Workspace* ws) {
+    if (!ws) return;
+    const uint32_t wm = wave_max_u32(lane_bits);
+    if ((threadIdx.x & 63) == 0 && wm != 0u)
+        __hip_atomic_fetch_max(&ws->slot[blockIdx.x % kMaxSlots].bits, wm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// fp8 epilogue of one wave for 32 x 32 accumulator blocks (layout as store_wave_tile); returns the lane's max|r| bits
+template <int F, int MI, int NJ>
+__device__ __forceinline__ uint32_t store_wave_tile_fp8(const v16f (&acc)[MI][NJ], uint8_t* __restrict__ D,
+                                                        uint8_t* __restrict__ Dt, float alpha, float scale_d, bool slow,
+                                                        int M, int N, int m_base, int n_base, int lane) {
+    uint32_t amax = 0;
+    const bool d_vec = (N & 3) == 0;   // rows of D start 4-byte aligned (the launcher checks D itself)
+    const bool t_vec = (M & 3) == 0 && (reinterpret_cast<uintptr_t>(Dt) & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+        const int m = m_base + i * 32 + (lane & 31);
+        const int mq = m & ~3;   // first row of this lane's quad
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n_base + j * 32 + g * 8 + (lane >> 5) * 4;
+                const uint32_t w = quant4<F>(acc[i][j][g * 4 + 0] * alpha, acc[i][j][g * 4 + 1] * alpha,
+                                             acc[i][j][g * 4 + 2] * alpha, acc[i][j][g * 4 + 3] * alpha, scale_d, slow, amax);
+                if (m < M && n < N) store_bytes4(D + (int64_t)m * N + n, w, d_vec, N - n);
+                if (Dt) {   // uniform
+                    const uint32_t t = quad_transpose_bytes(w, lane);
+                    const int nt = n + (lane & 3);
+                    if (nt < N && mq < M) store_bytes4(Dt + (int64_t)nt * M + mq, t, t_vec, M - mq);
+                }
+            }
+        }
+    }
+    return amax;
+}
+
 }  // namespace ntfp8

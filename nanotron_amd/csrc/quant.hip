@@ -157,38 +157,10 @@ __device__ __forceinline__ EpiloguePrefetch prefetch_epilogue(const ScalarIO& io
     return p;
 }
 
-template <int THREADS>
-__device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, const ScalarIO& io, int mode,
-                                            const EpiloguePrefetch& pre) {
-    __shared__ uint32_t s_part[THREADS / 64];
-    __shared__ bool s_last;
-    const uint32_t wm = wave_max_u32(m_f32bits);
-    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = wm;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t bm = 0;
-#pragma unroll
-        for (int i = 0; i < THREADS / 64; ++i) bm = s_part[i] > bm ? s_part[i] : bm;
-        // Two-level arrival count: a block publishes into the slot of its group and draws a ticket there; the
-        // last block of a group draws a ticket of the launch.  All blocks finish at about the same time, and
-        // their atomics on one address would queue one behind the other.
-        const uint32_t grp = blockIdx.x % kMaxSlots;
-        const uint32_t old = __hip_atomic_fetch_max(&ws->slot[grp].bits, bm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("s_waitcnt vmcnt(0)" ::"v"(old) : "memory");   // the max is in place before the ticket is drawn
-        const uint32_t in_group = (gridDim.x - grp + kMaxSlots - 1) / kMaxSlots;
-        const uint32_t t = __hip_atomic_fetch_add(&ws->slot[grp].ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        bool last = false;
-        if (t == in_group - 1) {
-            const uint32_t groups = gridDim.x < (uint32_t)kMaxSlots ? gridDim.x : (uint32_t)kMaxSlots;
-            const uint32_t t2 = __hip_atomic_fetch_add(&ws->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            last = (t2 == groups - 1);
-        }
-        s_last = last;
-    }
-    __syncthreads();
-    // The epilogue runs on the first wave of the block that drew the last ticket: every global access
-    // below is one round trip for the whole wave instead of one per history entry.
-    if (!s_last || threadIdx.x >= 64) return;
+// Bookkeeping of one launch, run by one wave (lanes 0..63 of a workgroup) once every workgroup's maximum is in
+// the slots: amax, history roll, next scale; leaves the workspace zeroed.  Every global access is one round
+// trip for the whole wave instead of one per history entry.
+__device__ inline void finalize_wave(Workspace* ws, const ScalarIO& io, int mode, const EpiloguePrefetch& pre) {
     const int lane = threadIdx.x;
     uint32_t bits = 0;
     if (lane < kMaxSlots) bits = __hip_atomic_load(&ws->slot[lane].bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -234,6 +206,46 @@ __device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, c
         __hip_atomic_store(&ws->slot[lane].bits, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(&ws->slot[lane].ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+}
+
+template <int THREADS>
+__device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, const ScalarIO& io, int mode,
+                                            const EpiloguePrefetch& pre) {
+    __shared__ uint32_t s_part[THREADS / 64];
+    __shared__ bool s_last;
+    const uint32_t wm = wave_max_u32(m_f32bits);
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = wm;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t bm = 0;
+#pragma unroll
+        for (int i = 0; i < THREADS / 64; ++i) bm = s_part[i] > bm ? s_part[i] : bm;
+        // Two-level arrival count: a block publishes into the slot of its group and draws a ticket there; the
+        // last block of a group draws a ticket of the launch.  All blocks finish at about the same time, and
+        // their atomics on one address would queue one behind the other.
+        const uint32_t grp = blockIdx.x % kMaxSlots;
+        const uint32_t old = __hip_atomic_fetch_max(&ws->slot[grp].bits, bm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::"v"(old) : "memory");   // the max is in place before the ticket is drawn
+        const uint32_t in_group = (gridDim.x - grp + kMaxSlots - 1) / kMaxSlots;
+        const uint32_t t = __hip_atomic_fetch_add(&ws->slot[grp].ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        bool last = false;
+        if (t == in_group - 1) {
+            const uint32_t groups = gridDim.x < (uint32_t)kMaxSlots ? gridDim.x : (uint32_t)kMaxSlots;
+            const uint32_t t2 = __hip_atomic_fetch_add(&ws->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last = (t2 == groups - 1);
+        }
+        s_last = last;
+    }
+    __syncthreads();
+    // the epilogue runs on the first wave of the block that drew the last ticket
+    if (!s_last || threadIdx.x >= 64) return;
+    finalize_wave(ws, io, mode, pre);
+}
+
+// The same bookkeeping for maxima that another kernel (the fp8-output GEMM epilogue) left in the slots.
+__global__ __launch_bounds__(64) void amax_finalize_kernel(Workspace* ws, ScalarIO io) {
+    const EpiloguePrefetch pre = prefetch_epilogue(io, kModeDelayed);
+    finalize_wave(ws, io, kModeDelayed, pre);
 }
 
 __device__ __forceinline__ bool degenerate_scale(float s) {
@@ -554,6 +566,11 @@ int run_transpose(const void* in, int64_t rows, int64_t cols, void* out, hipStre
     if (tiles > 0x7fffffff) return NTFP8_ERR_SIZE;
     hipLaunchKernelGGL(transpose_kernel, dim3((int)tiles), dim3(kThreads), 0, st, static_cast<const uint8_t*>(in), rows,
                        cols, static_cast<uint8_t*>(out));
+    return check_launch();
+}
+
+int run_amax_finalize(Workspace* ws, const ScalarIO& io, hipStream_t st) {
+    hipLaunchKernelGGL(amax_finalize_kernel, dim3(1), dim3(64), 0, st, ws, io);
     return check_launch();
 }
 

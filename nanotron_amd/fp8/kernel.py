@@ -1,12 +1,13 @@
-from typing import Optional
+from typing import Optional, Union
 
 import torch
 
 from nanotron_amd import _native as nt
 from nanotron_amd.fp8.dtypes import DTypes
-from nanotron_amd.fp8.tensor import FP8Tensor
+from nanotron_amd.fp8.tensor import DelayedScaling, FP8Tensor
 
 _FMT = {DTypes.FP8E4M3: nt.E4M3, DTypes.FP8E5M2: nt.E5M2}
+_OUT_FMT = {DTypes.FP8E4M3: nt.OUT_E4M3, DTypes.FP8E5M2: nt.OUT_E5M2}
 
 
 def _gemm_nt(a: FP8Tensor, b: FP8Tensor, out_dtype: torch.dtype, accumulate_into: Optional[torch.Tensor]):
@@ -31,6 +32,54 @@ def _gemm_nt(a: FP8Tensor, b: FP8Tensor, out_dtype: torch.dtype, accumulate_into
                                out.data_ptr(), nt.TORCH_TO_NT[out.dtype], M, N, K, acc, nt.stream_ptr(dev)),
              "ntfp8_gemm")
     return out
+
+
+def _gemm_nt_fp8(a: FP8Tensor, b: FP8Tensor, dtype: DTypes, state: Optional[DelayedScaling],
+                 with_transpose: bool) -> FP8Tensor:
+    """FP8Tensor(_gemm_nt(a, b, float32), dtype, state=state, with_transpose=with_transpose), bit for bit, with the
+    fp32 result never written to memory: the GEMM epilogue casts with the scale `state` holds from earlier steps,
+    leaves max|result| behind, and a one-wave kernel turns that into amax, history roll and next scale.
+
+    The amax of a GEMM result is not known before the GEMM has run, so a step without a held scale (no `state`, or
+    one that has not seen a usable amax yet) goes the long way: fp32 result, then the ordinary quantisation."""
+    from nanotron_amd.fp8.meta import FP8Meta
+
+    assert dtype in _OUT_FMT, f"{dtype} is not an FP8 format"
+    if state is None or not state.initialised:
+        return FP8Tensor(_gemm_nt(a, b, torch.float32, None), dtype, state=state, with_transpose=with_transpose)
+    assert state.dtype == dtype, "delayed-scaling state was created for another format"
+    assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[1], (tuple(a.shape), tuple(b.shape))
+    M, K = a.shape
+    N = b.shape[0]
+    dev = a.device
+    assert state._buf.device == dev
+    if not a.is_contiguous():
+        a = a.contiguous()
+    if not b.is_contiguous():
+        b = b.contiguous()
+    ma, mb = a.fp8_meta, b.fp8_meta
+    out = torch.empty((M, N), dtype=torch.uint8, device=dev)
+    out_t = torch.empty((N, M), dtype=torch.uint8, device=dev) if with_transpose else None
+    scalars = torch.empty(2, dtype=torch.float32, device=dev)  # [amax, scale used]
+    ws, st = nt.workspace_and_stream(dev)
+    state_p = state._buf.data_ptr()  # [scale, hist[0..H-1]]
+    d = (nt.GemmDesc * 1)()
+    d[0].A, d[0].scale_a, d[0].B, d[0].scale_b, d[0].D = (a.data_ptr(), ma.scale.data_ptr(), b.data_ptr(),
+                                                          mb.scale.data_ptr(), out.data_ptr())
+    d[0].M, d[0].N, d[0].K = M, N, K
+    d[0].fmt_a, d[0].fmt_b, d[0].d_dtype, d[0].accumulate = _FMT[ma.dtype], _FMT[mb.dtype], _OUT_FMT[dtype], 0
+    d[0].scale_d, d[0].D_t, d[0].amax_workspace = state_p, nt.ptr(out_t), ws.data_ptr()
+    nt.check(nt.lib.ntfp8_gemm_batch(d, 1, st), "ntfp8_gemm_batch")
+    nt.check(nt.lib.ntfp8_amax_finalize(ws.data_ptr(), _FMT[dtype], state.margin, state_p, state_p + 4, state.history_len,
+                                        scalars.data_ptr(), scalars.data_ptr() + 4, st), "ntfp8_amax_finalize")
+    meta = FP8Meta(scalars[0], scalars[1], dtype)
+    obj = torch.Tensor._make_subclass(FP8Tensor, out)
+    obj.fp8_meta = meta
+    if out_t is not None:
+        t = torch.Tensor._make_subclass(FP8Tensor, out_t)
+        t.fp8_meta = meta
+        obj._transposed = t
+    return obj
 
 
 def _gemm_nt_batch(problems):
@@ -95,8 +144,10 @@ def fp8_matmul_kernel(
     transpose_b: bool,
     use_split_accumulator: bool,
     *,
-    out_dtype: Optional[torch.dtype] = None,
+    out_dtype: Union[torch.dtype, DTypes, None] = None,
     accumulate_into: Optional[torch.Tensor] = None,
+    out_state: Optional[DelayedScaling] = None,
+    out_with_transpose: bool = False,
 ) -> torch.Tensor:
     """D = op_b(B) . op_a(A) * (1/scale_a)(1/scale_b), op_x(X) = X^T if transpose_x else X
     (reference: src/nanotron/fp8/kernel.py:9-70; the operator meaning follows from its fixed
@@ -106,10 +157,16 @@ def fp8_matmul_kernel(
 
     `use_split_accumulator` selects cuBLASLt's slower, more accurate accumulation on Hopper; CDNA4
     matrix cores always accumulate in fp32, so it is accepted and ignored.
-    `accumulate_into` (fp32, contiguous) receives D added in place before any rounding."""
+    `accumulate_into` (fp32, contiguous) receives D added in place before any rounding.
+    `out_dtype=DTypes.FP8E4M3 / FP8E5M2` returns D as an FP8Tensor ("return an fp8 tensor as output", the TODO at
+    src/nanotron/fp8/linear.py:63-64), quantised with the delayed-scaling state `out_state` in the GEMM's epilogue
+    and, with `out_with_transpose`, carrying its transposed copy."""
     assert mat_a.device != torch.device("cpu") and mat_b.device != torch.device("cpu"), \
         "The tensors must be on a CUDA device in order to use the FP8 kernel!!"
     assert hasattr(mat_a, "fp8_meta") and hasattr(mat_b, "fp8_meta"), "operands must be FP8Tensors"
     a_ = mat_a if transpose_a else mat_a.transposed()  # kernel.py:43
     b_ = mat_b.transposed() if transpose_b else mat_b  # kernel.py:44
+    if isinstance(out_dtype, DTypes):
+        assert accumulate_into is None, "an fp8 output cannot accumulate"
+        return _gemm_nt_fp8(b_, a_, out_dtype, out_state, out_with_transpose)
     return _gemm_nt(b_, a_, out_dtype or torch.float32, accumulate_into)

@@ -25,18 +25,26 @@ class FP8Linear(nn.Linear):
 
     Positional signature as the reference.  Keyword-only extensions, all defaulting to the
     reference's behaviour: `dtype` (of the master weight and bias, as nn.Linear's), `out_dtype`
-    (None = fp32 output, kernel.py:24,28), `delayed_scaling`
+    (None = fp32 output, kernel.py:24,28; `DTypes.FP8E4M3` / `FP8E5M2` = the output is returned as an
+    FP8Tensor, the TODO at linear.py:63-64: forward only, no bias, quantised in the GEMM epilogue with the
+    delayed-scaling role "output", its transposed copy included if `fp8_output_transpose`), `delayed_scaling`
     (False = scale every tensor from its own amax), `amax_history_len`, `margin`,
     `accumulate_grad` (False = `weight.grad` is overwritten each backward, linear.py:110; True =
     the wgrad GEMM adds into the existing fp32 gradient in its epilogue).  With a bf16 / fp16
     master weight the fp32 weight gradient is stored as `weight.main_grad` instead of `.grad`."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, device: Optional[torch.device] = None,
-                 *, dtype: Optional[torch.dtype] = None, out_dtype: Optional[torch.dtype] = None,
+                 *, dtype: Optional[torch.dtype] = None, out_dtype: Union[torch.dtype, DTypes, None] = None,
                  delayed_scaling: bool = False, amax_history_len: int = 16, margin: int = 0,
-                 accumulate_grad: bool = False):
+                 accumulate_grad: bool = False, fp8_output_transpose: bool = False):
         super().__init__(in_features, out_features, bias, device, dtype)
+        if isinstance(out_dtype, DTypes):
+            if out_dtype not in (DTypes.FP8E4M3, DTypes.FP8E5M2):
+                raise ValueError(f"{out_dtype} is not an FP8 format")
+            if bias:
+                raise ValueError("an fp8 output is quantised inside the GEMM, before a bias could be added: use bias=False")
         self.out_dtype = out_dtype
+        self.fp8_output_transpose = fp8_output_transpose
         self.accumulate_grad = accumulate_grad
         self.scaling = None
         self._weight_ready = None
@@ -66,6 +74,8 @@ class FP8Linear(nn.Linear):
                     "weight": DelayedScaling(DTypes.FP8E4M3, amax_history_len, margin, dev),
                     "output_grad": DelayedScaling(DTypes.FP8E5M2, amax_history_len, margin, dev),
                 }
+                if isinstance(out_dtype, DTypes):
+                    self.scaling["output"] = DelayedScaling(out_dtype, amax_history_len, margin, dev)
 
     @torch.no_grad()
     def requantize_weight(self, stream: Optional[torch.cuda.Stream] = None) -> None:
@@ -184,6 +194,15 @@ class _FP8Matmul(torch.autograd.Function):
         out_dtype = module.out_dtype or torch.float32
 
         # FP8Tensor of the weight, not the FP8Parameter (linear.py:81-84)
+        if isinstance(out_dtype, DTypes):
+            # [tokens, out_features] whatever the input's leading dimensions: what the next layer's GEMM consumes
+            output = fp8_matmul_kernel(
+                mat_a=weight.data, transpose_a=True, mat_b=input, transpose_b=False, use_split_accumulator=False,
+                out_dtype=out_dtype, out_state=scaling["output"] if scaling else None,
+                out_with_transpose=module.fp8_output_transpose,
+            )
+            ctx.mark_non_differentiable(output)
+            return output, phony
         output = fp8_matmul_kernel(
             mat_a=weight.data, transpose_a=True, mat_b=input, transpose_b=False, use_split_accumulator=False,
             out_dtype=out_dtype,
