@@ -57,6 +57,9 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--weight-stream", action="store_true",
                    help="re-quantise the weights on a second stream (measured: no gain, the GEMMs are power-bound)")
+    p.add_argument("--transposed-copies", action="store_true",
+                   help="quantise weights and inputs together with transposed copies and run the backward GEMMs on "
+                        "those (the reference's way) instead of letting the GEMM read the tensors as they are")
     p.add_argument("--kernel-reps", type=int, default=0,
                    help="also time each GEMM shape in isolation with this many back-to-back launches (0 = skip)")
     return p.parse_args()
@@ -348,6 +351,10 @@ def main():
         sys.exit(2)
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
+    if args.transposed_copies:
+        import nanotron_amd.fp8.kernel as K
+
+        K.READ_B_TRANSPOSED = False
 
     if args.workload == "probe":
         probe(device)

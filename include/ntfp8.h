@@ -129,6 +129,13 @@ typedef struct ntfp8_gemm_desc {
     const float* scale_d;   /* device scalar: the result is multiplied by it before the cast */
     void* D_t;              /* NULL, or [N, M] bytes: the transposed copy of D */
     void* amax_workspace;   /* NULL, or NTFP8_WORKSPACE_BYTES, all zero: collects max|result| */
+    /* != 0: B points to the [K, N] row-major bytes of B's transpose, i.e. to a tensor whose row index is the
+     * reduction index.  That is what the backward GEMMs of a linear layer have at hand (dgrad: W[N_out, K_in]
+     * reduces over N_out; wgrad: X[tokens, K_in] reduces over tokens; src/nanotron/fp8/linear.py:104-109), and
+     * where the reference calls tex.fp8_transpose first (src/nanotron/fp8/kernel.py:43) this library reads the
+     * tensor as it is.  Served for N a multiple of 16, M and N above 128, K at least 256, operands below 2 GiB
+     * and outputs other than fp8; anything else returns NTFP8_ERR_UNSUPPORTED (transpose B and pass 0). */
+    int b_transposed;
 } ntfp8_gemm_desc;
 #define NTFP8_MAX_BATCH 64
 int ntfp8_gemm_batch(const ntfp8_gemm_desc* problems, int count, void* stream);

@@ -37,7 +37,7 @@ class GemmDesc(ctypes.Structure):
     _fields_ = [("A", _vp), ("scale_a", _vp), ("B", _vp), ("scale_b", _vp), ("D", _vp),
                 ("M", _i64), ("N", _i64), ("K", _i64),
                 ("fmt_a", _i), ("fmt_b", _i), ("d_dtype", _i), ("accumulate", _i),
-                ("scale_d", _vp), ("D_t", _vp), ("amax_workspace", _vp)]
+                ("scale_d", _vp), ("D_t", _vp), ("amax_workspace", _vp), ("b_transposed", _i)]
 
 
 SIGNATURES = {

@@ -73,7 +73,8 @@ int check_gemm(const ntfp8_gemm_desc& p, GemmDesc* g) {
     const size_t db = (size_t)mn * dtype_size(p.d_dtype);
     if (overlap(p.A, (size_t)mk, p.D, db) || overlap(p.B, (size_t)nk, p.D, db)) return NTFP8_ERR_ALIAS;
     *g = GemmDesc{p.A, p.fmt_a, p.scale_a, p.B, p.fmt_b, p.scale_b, p.D, p.d_dtype, (int)M, (int)N, (int)K, p.accumulate ? 1 : 0,
-                  nullptr, nullptr, nullptr};
+                  nullptr, nullptr, nullptr, p.b_transposed ? 1 : 0};
+    if (p.b_transposed && fp8_out) return NTFP8_ERR_UNSUPPORTED;
     if (fp8_out) {
         if (!is_aligned(p.scale_d, 4) || (p.amax_workspace && !is_aligned(p.amax_workspace, 4))) return NTFP8_ERR_ALIGN;
         if (p.D_t && (overlap(p.A, (size_t)mk, p.D_t, db) || overlap(p.B, (size_t)nk, p.D_t, db) || overlap(p.D, db, p.D_t, db)))
@@ -217,7 +218,7 @@ int ntfp8_transpose(const void* in, int64_t rows, int64_t cols, void* out, void*
 int ntfp8_gemm(const void* A, int fmt_a, const float* scale_a, const void* B, int fmt_b, const float* scale_b, void* D,
                int d_dtype, int64_t M, int64_t N, int64_t K, int accumulate, void* stream) {
     if (is_fp8_out(d_dtype)) return NTFP8_ERR_UNSUPPORTED;   // fp8 outputs carry more arguments: ntfp8_gemm_batch
-    const ntfp8_gemm_desc p = {A, scale_a, B, scale_b, D, M, N, K, fmt_a, fmt_b, d_dtype, accumulate, nullptr, nullptr, nullptr};
+    const ntfp8_gemm_desc p = {A, scale_a, B, scale_b, D, M, N, K, fmt_a, fmt_b, d_dtype, accumulate, nullptr, nullptr, nullptr, 0};
     GemmDesc g;
     const int rc = check_gemm(p, &g);
     if (rc) return rc;

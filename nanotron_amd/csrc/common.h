@@ -143,6 +143,7 @@ struct GemmDesc {
     const float* sd;
     void* Dt;
     void* ws;
+    int tb;   // B is given as [K, N] row-major (its transpose)
 };
 
 __host__ __device__ inline bool is_fp8_out(int d_dtype) { return d_dtype == NTFP8_OUT_E4M3 || d_dtype == NTFP8_OUT_E5M2; }

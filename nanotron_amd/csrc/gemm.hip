@@ -159,14 +159,14 @@ __global__ void gemm_nt_naive_kernel(const uint8_t* __restrict__ A, const uint8_
 }
 
 // ---------------------------------------------------------------------------------------------
-enum GemmPath { kPathNaive = 0, kPathSmall = 1, kPathBig = 2 };
+enum GemmPath { kPathNone = -1, kPathNaive = 0, kPathSmall = 1, kPathBig = 2 };
 
 // which kernel serves a problem
 static int path_of(const GemmDesc& g) {
     const bool aligned16 = (g.K % 16 == 0) &&
                            ((reinterpret_cast<uintptr_t>(g.A) | reinterpret_cast<uintptr_t>(g.B)) & 15) == 0 &&
                            (reinterpret_cast<uintptr_t>(g.D) & 15) == 0;
-    if (!aligned16) return kPathNaive;
+    if (!aligned16) return g.tb ? kPathNone : kPathNaive;
     // the big kernel addresses its operands with 32-bit buffer offsets and wants enough tiles to matter
     const bool fits32 = (int64_t)(g.M + 256) * g.K < (1LL << 31) && (int64_t)(g.N + kBigN) * g.K < (1LL << 31);
     const bool worth = g.M > kBM && g.N > kBN && g.K >= 2 * kBK;
@@ -174,13 +174,15 @@ static int path_of(const GemmDesc& g) {
     const bool fp8_ok = !is_fp8_out(g.d_dtype) ||
                         (g.N % 16 == 0 && g.M % 4 == 0 && (int64_t)g.M * g.N < (1LL << 32) - 16 &&
                          (reinterpret_cast<uintptr_t>(g.Dt) & 15) == 0);
+    // a B operand given as [K, N] is loaded in 16-byte pieces of its rows; only the big kernel reads it
+    if (g.tb) return (g.N % 16 == 0 && fits32 && worth && !is_fp8_out(g.d_dtype)) ? kPathBig : kPathNone;
     return (fits32 && worth && fp8_ok) ? kPathBig : kPathSmall;
 }
 
 // One launch (plus one for the half-tile tail) of the big kernel over up to kBigMaxProblems problems of the
 // same operand formats.  Tiles are listed problem by problem, longest K first: the long tiles start together and
 // the shorter ones fill the rounds behind them.
-template <int FA, int FB, bool kFp8Out>
+template <int FA, int FB, bool kFp8Out, bool kBT>
 static int launch_big(const GemmDesc* const* g, int n, hipStream_t st) {
     int order[kBigMaxProblems];
     for (int i = 0; i < n; ++i) order[i] = i;
@@ -217,9 +219,9 @@ static int launch_big(const GemmDesc* const* g, int n, hipStream_t st) {
     L.full_blocks = tiles - L.tail_tiles;
     L.round_size = cu_count();
     if (L.full_blocks > 0)
-        hipLaunchKernelGGL((gemm_nt_big_kernel<FA, FB, 8, kFp8Out>), dim3(L.full_blocks), dim3(kBigThreads), 0, st, L);
+        hipLaunchKernelGGL((gemm_nt_big_kernel<FA, FB, 8, kFp8Out, kBT>), dim3(L.full_blocks), dim3(kBigThreads), 0, st, L);
     if (L.tail_tiles > 0)
-        hipLaunchKernelGGL((gemm_nt_big_kernel<FA, FB, 4, kFp8Out>), dim3(2 * L.tail_tiles), dim3(kBigThreads), 0, st, L);
+        hipLaunchKernelGGL((gemm_nt_big_kernel<FA, FB, 4, kFp8Out, kBT>), dim3(2 * L.tail_tiles), dim3(kBigThreads), 0, st, L);
     return hipGetLastError() == hipSuccess ? NTFP8_OK : NTFP8_ERR_LAUNCH;
 }
 
@@ -242,8 +244,11 @@ static int launch_small(const GemmDesc& g, int path, hipStream_t st) {
 
 template <int FA, int FB>
 static int dispatch_fmt(const GemmDesc* const* g, int n, int path, hipStream_t st) {
-    if (path == kPathBig)
-        return is_fp8_out(g[0]->d_dtype) ? launch_big<FA, FB, true>(g, n, st) : launch_big<FA, FB, false>(g, n, st);
+    if (path == kPathNone) return NTFP8_ERR_UNSUPPORTED;
+    if (path == kPathBig) {
+        if (g[0]->tb) return launch_big<FA, FB, false, true>(g, n, st);
+        return is_fp8_out(g[0]->d_dtype) ? launch_big<FA, FB, true, false>(g, n, st) : launch_big<FA, FB, false, false>(g, n, st);
+    }
     const GemmDesc& d = *g[0];   // the small kernels take one problem
     if (d.d_dtype == NTFP8_F32)
         return d.accumulate ? launch_small<FA, FB, NTFP8_F32, true>(d, path, st)
@@ -280,7 +285,7 @@ int run_gemm_batch(const GemmDesc* g, int n, hipStream_t st) {
         if (path == kPathBig) {
             for (int j = i + 1; j < n && cnt < kBigMaxProblems; ++j)
                 if (!done[j] && g[j].fmt_a == g[i].fmt_a && g[j].fmt_b == g[i].fmt_b && path_of(g[j]) == kPathBig &&
-                    is_fp8_out(g[j].d_dtype) == is_fp8_out(g[i].d_dtype)) {
+                    is_fp8_out(g[j].d_dtype) == is_fp8_out(g[i].d_dtype) && g[j].tb == g[i].tb) {
                     group[cnt++] = &g[j];
                     done[j] = true;
                 }

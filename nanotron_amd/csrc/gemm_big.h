@@ -234,7 +234,16 @@ struct BigLaunch {
 // register set and copies them back and forth inside the K loop.
 // kFp8Out: every problem of the launch has an fp8 output (a kernel of its own: the other outputs' code stays as
 // the register allocator likes it).
-template <int FA, int FB, int MI, bool kFp8Out = false>
+// kBT: the B operands are given transposed, as [K, N] row-major bytes (what a caller has when the reduction index is
+// the row index of its tensor: W for dgrad, X for wgrad).  A K-tile of such an operand lies in LDS as it lies in
+// memory, 128 rows of k with 256 bytes of n each, and the 16 x 128 fragments are gathered with the transposing
+// LDS read DS_READ_B64_TR_B8: within 16 lanes, lane 2 u supplies the address of 8 bytes that lanes 0-7 receive one
+// byte each of (byte i to lane i, as their byte u), lane 2 u + 1 the same for lanes 8-15.  With lane 2 u on row
+// k0 + u, columns c .. c + 7, and lane 2 u + 1 on the same row, columns c + 8 .. c + 15, lane r receives k0 .. k0 + 7
+// of column c + r: a quarter of its fragment.  16-byte chunk c of row k is stored at chunk
+// c ^ ((k mod 8) | 8 (k / 32 mod 2)), so that the 8 rows one read touches (and the two 16-lane groups that go
+// through LDS together) use different banks.
+template <int FA, int FB, int MI, bool kFp8Out = false, bool kBT = false>
 __global__ __launch_bounds__(MI == 8 ? kBigThreads : 2 * kBigThreads)
 void gemm_nt_big_kernel(const BigLaunch L) {
     // whole tiles: 2 stages of 64 KB; half tiles: 3 stages of 48 KB (their loads go straight to LDS and need the
@@ -311,8 +320,20 @@ void gemm_nt_big_kernel(const BigLaunch L) {
         for (int i = 0; i < LA; ++i)   // rows >= M fall past the descriptor: zeros
             a_off[i] = (uint32_t)(m0 + (wave + kBigWaves * i) * 8 + (lane >> 3)) * (uint32_t)K + ld_kc;
 #pragma unroll
-        for (int i = 0; i < LB; ++i)
-            b_off[i] = (uint32_t)(n0 + (wave + kBigWaves * i) * 8 + (lane >> 3)) * (uint32_t)K + ld_kc;
+        for (int i = 0; i < LB; ++i) {
+            if constexpr (kBT) {
+                // a wave-level load fills 4 rows of k (lane / 16) with 16 chunks of n (lane % 16) each; rows k >= K fall
+                // past the descriptor (zeros); chunks past N wrap into the next row and only reach outputs that are
+                // never stored
+                const int k = (wave + kBigWaves * i) * 4 + (lane >> 4);
+                const int chunk = (lane & 15) ^ ((k & 7) | (((k >> 5) & 1) << 3));
+                b_off[i] = (uint32_t)k * (uint32_t)N + (uint32_t)(n0 + chunk * 16);
+            } else {
+                b_off[i] = (uint32_t)(n0 + (wave + kBigWaves * i) * 8 + (lane >> 3)) * (uint32_t)K + ld_kc;
+            }
+        }
+        // byte distance between K-tiles in memory
+        const int a_step = kBK, b_step = kBT ? kBK * N : kBK;
 
         v4f acc[MI][kBigNJ];
 #pragma unroll
@@ -324,9 +345,9 @@ void gemm_nt_big_kernel(const BigLaunch L) {
         auto issue = [&](int ktile, int l) {
             const int s = ktile % NS;
             if (l < LA)
-                lds_load16(ra, (lds_ptr)(uintptr_t)&sA[s][(wave + kBigWaves * l) * 1024], a_off[l], ktile * kBK);
+                lds_load16(ra, (lds_ptr)(uintptr_t)&sA[s][(wave + kBigWaves * l) * 1024], a_off[l], ktile * a_step);
             else
-                lds_load16(rb, (lds_ptr)(uintptr_t)&sB[s][(wave + kBigWaves * (l - LA)) * 1024], b_off[l - LA], ktile * kBK);
+                lds_load16(rb, (lds_ptr)(uintptr_t)&sB[s][(wave + kBigWaves * (l - LA)) * 1024], b_off[l - LA], ktile * b_step);
         };
         // Called once, before the first load of the last K-tile is queued (no other tile is loaded after it):
         // lanes whose chunk lies at k >= K get an offset past the descriptor and so read zeros.
@@ -334,8 +355,10 @@ void gemm_nt_big_kernel(const BigLaunch L) {
             if (tail_dead) {
 #pragma unroll
                 for (int i = 0; i < LA; ++i) a_off[i] = 0xfffffff0u;
+                if constexpr (!kBT) {
 #pragma unroll
-                for (int i = 0; i < LB; ++i) b_off[i] = 0xfffffff0u;
+                    for (int i = 0; i < LB; ++i) b_off[i] = 0xfffffff0u;
+                }
             }
         };
 
@@ -349,8 +372,26 @@ void gemm_nt_big_kernel(const BigLaunch L) {
         auto rd_a = [&](int s, int i, int h) -> v4i {
             return *reinterpret_cast<const v4i*>(&sA[s][(h ? a_rd1 : a_rd0) + i * 2048]);
         };
+        // transposed B: lane u of a 16-lane group (which serves k 32 (lane / 16) .. + 31) addresses row k0 + u / 2,
+        // half u % 2 of the block's 16-byte chunk; quarter t of the fragment is k0 = 32 (lane / 16) + 8 t
+        const int bt_row = (lane & 15) >> 1;
+        const int bt_base = ((lane >> 4) * 32 + bt_row) * 256 + ((((wave & 1) ^ ((lane >> 4) & 1))) << 7) + (lane & 1) * 8;
+        const int bt_x = bt_row << 4;
         auto rd_b = [&](int s, int j, int h) -> v4i {
-            return *reinterpret_cast<const v4i*>(&sB[s][(h ? b_rd1 : b_rd0) + j * 2048]);
+            if constexpr (kBT) {
+                typedef int v2i __attribute__((ext_vector_type(2)));
+                typedef __attribute__((address_space(3))) v2i* tr_ptr;
+                // (address-space cast, not a round trip through an integer: the compiler must see that these reads
+                // come from sB, or it waits for every direct-to-LDS load in flight before each of them)
+                int x = bt_x;
+                asm volatile("" : "+v"(x));   // recomputed at every use: eight block offsets kept across the K loop do not fit
+                uint8_t* p = &sB[s][bt_base + ((j << 4) ^ x) + h * (2 * 8 * 256)];
+                const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((tr_ptr)p);
+                const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((tr_ptr)(p + 8 * 256));
+                return (v4i){lo.x, lo.y, hi.x, hi.y};
+            } else {
+                return *reinterpret_cast<const v4i*>(&sB[s][(h ? b_rd1 : b_rd0) + j * 2048]);
+            }
         };
         auto frag = [](const v4i (&x)[2]) -> v8i { return (v8i){x[0].x, x[0].y, x[0].z, x[0].w, x[1].x, x[1].y, x[1].z, x[1].w}; };
 
@@ -444,7 +485,7 @@ void gemm_nt_big_kernel(const BigLaunch L) {
             v4i g[NL];
             const int wr_lane = wave * 1024 + lane * 16;   // a wave-level load covers 1 KB of a stage: 16 bytes per lane
             auto request = [&](int ktile, int l) {
-                g[l] = l < LA ? reg_load16(ra, a_off[l], ktile * kBK) : reg_load16(rb, b_off[l - LA], ktile * kBK);
+                g[l] = l < LA ? reg_load16(ra, a_off[l], ktile * a_step) : reg_load16(rb, b_off[l - LA], ktile * b_step);
             };
             auto deposit = [&](int s, int l) {
                 if (l < LA) *reinterpret_cast<v4i*>(&sA[s][wr_lane + l * (kBigWaves * 1024)]) = g[l];

@@ -82,17 +82,39 @@ def _gemm_nt_fp8(a: FP8Tensor, b: FP8Tensor, dtype: DTypes, state: Optional[Dela
     return obj
 
 
+# Module switch: False makes every GEMM use materialised transposed copies (the reference's way, kernel.py:43-44).
+READ_B_TRANSPOSED = True
+
+
+def b_transposed_supported(M: int, N: int, K: int) -> bool:
+    """Whether the library reads the B operand of D[M,N] = A[M,K] . B[N,K]^T from its transpose, a [K, N] tensor
+    (`ntfp8_gemm_desc.b_transposed`): the condition stated in include/ntfp8.h."""
+    return (READ_B_TRANSPOSED and N % 16 == 0 and K % 16 == 0 and M > 128 and N > 128 and K >= 256
+            and (M + 256) * K < 2 ** 31 and (N + 256) * K < 2 ** 31)
+
+
+def needs_transposed_copy(rows: int, cols: int, other: int = 4096) -> bool:
+    """Whether a [rows, cols] fp8 tensor that a backward GEMM reduces over its rows (the weight in dgrad, the input in
+    wgrad; src/nanotron/fp8/linear.py:104-109) should be quantised together with its transposed copy: only if the
+    library cannot read it as it is.  `other` is the GEMM's third dimension (tokens for the weight, out_features
+    for the input), assumed large when not known yet; a copy that turns out to be needed after all is made on demand."""
+    return not b_transposed_supported(other, cols, rows)
+
+
 def _gemm_nt_batch(problems):
-    """Several independent `_gemm_nt` problems, given as tuples (a, b, out_dtype, accumulate_into), in one call of
-    the library: GEMMs with the same operand formats share launches.  Returns the outputs in order."""
+    """Several independent `_gemm_nt` problems, given as tuples (a, b, out_dtype, accumulate_into[, b_transposed]),
+    in one call of the library: GEMMs with the same operand formats share launches.  With `b_transposed` the
+    tensor `b` is the [K, N] transpose of the operand.  Returns the outputs in order."""
     descs = (nt.GemmDesc * len(problems))()
     outs, keep = [], []
     dev = problems[0][0].device
-    for d, (a, b, out_dtype, accumulate_into) in zip(descs, problems):
-        assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[1], (tuple(a.shape), tuple(b.shape))
+    for d, prob in zip(descs, problems):
+        a, b, out_dtype, accumulate_into = prob[:4]
+        bt = bool(prob[4]) if len(prob) > 4 else False
+        assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0 if bt else 1], (tuple(a.shape), tuple(b.shape), bt)
         assert a.device == dev and b.device == dev
         M, K = a.shape
-        N = b.shape[0]
+        N = b.shape[1 if bt else 0]
         if not a.is_contiguous():
             a = a.contiguous()
         if not b.is_contiguous():
@@ -107,6 +129,7 @@ def _gemm_nt_batch(problems):
         d.A, d.scale_a, d.B, d.scale_b, d.D = a.data_ptr(), ma.scale.data_ptr(), b.data_ptr(), mb.scale.data_ptr(), out.data_ptr()
         d.M, d.N, d.K = M, N, K
         d.fmt_a, d.fmt_b, d.d_dtype, d.accumulate = _FMT[ma.dtype], _FMT[mb.dtype], nt.TORCH_TO_NT[out.dtype], acc
+        d.b_transposed = 1 if bt else 0
         outs.append(out)
         keep.append((a, b))
     nt.check(nt.lib.ntfp8_gemm_batch(descs, len(problems), nt.stream_ptr(dev)), "ntfp8_gemm_batch")
@@ -114,13 +137,21 @@ def _gemm_nt_batch(problems):
 
 
 def _operands(mat_a: FP8Tensor, transpose_a: bool, mat_b: FP8Tensor, transpose_b: bool):
-    """(A, B) of the library's D = A . B^T for the reference's D = op_b(B) . op_a(A) (kernel.py:43-44)."""
+    """(A, B, b_transposed) of the library's D = A . B^T for the reference's D = op_b(B) . op_a(A) (kernel.py:43-44).
+
+    Where the reference transposes mat_a (tex.fp8_transpose, kernel.py:43) the library can read it as it is
+    (`b_transposed`): that is taken when mat_a carries no transposed copy yet and the shape qualifies; otherwise the
+    copy is used (and made, once, if it does not exist)."""
     assert mat_a.device != torch.device("cpu") and mat_b.device != torch.device("cpu"), \
         "The tensors must be on a CUDA device in order to use the FP8 kernel!!"
     assert hasattr(mat_a, "fp8_meta") and hasattr(mat_b, "fp8_meta"), "operands must be FP8Tensors"
-    a_ = mat_a if transpose_a else mat_a.transposed()
-    b_ = mat_b.transposed() if transpose_b else mat_b
-    return b_, a_
+    b_ = mat_b.transposed() if transpose_b else mat_b   # the library's A: always K-contiguous
+    if transpose_a:
+        return b_, mat_a, False
+    if getattr(mat_a, "_transposed", None) is None and mat_a.dim() == 2 and mat_a.is_contiguous() and \
+            b_transposed_supported(b_.shape[0], mat_a.shape[1], mat_a.shape[0]):
+        return b_, mat_a, True
+    return b_, mat_a.transposed(), False
 
 
 @torch.no_grad()
@@ -130,9 +161,9 @@ def fp8_matmul_pair(first: dict, second: dict):
     results as two calls; the library lets the two GEMMs share kernel launches."""
     probs = []
     for kw in (first, second):
-        A, B = _operands(kw["mat_a"], kw["transpose_a"], kw["mat_b"], kw["transpose_b"])
+        A, B, bt = _operands(kw["mat_a"], kw["transpose_a"], kw["mat_b"], kw["transpose_b"])
         acc = kw.get("accumulate_into")
-        probs.append((A, B, (kw.get("out_dtype") or torch.float32) if acc is None else torch.float32, acc))
+        probs.append((A, B, (kw.get("out_dtype") or torch.float32) if acc is None else torch.float32, acc, bt))
     return _gemm_nt_batch(probs)
 
 
@@ -164,9 +195,12 @@ def fp8_matmul_kernel(
     assert mat_a.device != torch.device("cpu") and mat_b.device != torch.device("cpu"), \
         "The tensors must be on a CUDA device in order to use the FP8 kernel!!"
     assert hasattr(mat_a, "fp8_meta") and hasattr(mat_b, "fp8_meta"), "operands must be FP8Tensors"
-    a_ = mat_a if transpose_a else mat_a.transposed()  # kernel.py:43
-    b_ = mat_b.transposed() if transpose_b else mat_b  # kernel.py:44
     if isinstance(out_dtype, DTypes):
         assert accumulate_into is None, "an fp8 output cannot accumulate"
+        a_ = mat_a if transpose_a else mat_a.transposed()  # kernel.py:43
+        b_ = mat_b.transposed() if transpose_b else mat_b  # kernel.py:44
         return _gemm_nt_fp8(b_, a_, out_dtype, out_state, out_with_transpose)
-    return _gemm_nt(b_, a_, out_dtype or torch.float32, accumulate_into)
+    A, B, bt = _operands(mat_a, transpose_a, mat_b, transpose_b)
+    if bt:
+        return _gemm_nt_batch([(A, B, out_dtype or torch.float32, accumulate_into, True)])[0]
+    return _gemm_nt(A, B, out_dtype or torch.float32, accumulate_into)

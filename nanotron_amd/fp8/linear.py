@@ -6,7 +6,7 @@ from torch import nn
 
 from nanotron_amd.fp8.constants import INITIAL_AMAX, INITIAL_SCALING_FACTOR
 from nanotron_amd.fp8.dtypes import DTypes
-from nanotron_amd.fp8.kernel import fp8_matmul_kernel, fp8_matmul_pair
+from nanotron_amd.fp8.kernel import fp8_matmul_kernel, fp8_matmul_pair, needs_transposed_copy
 from nanotron_amd.fp8.meta import FP8Meta
 from nanotron_amd.fp8.parameter import FP8Parameter
 from nanotron_amd.fp8.tensor import DelayedScaling, FP8Tensor, cast_with_scale, update_scaling_factor
@@ -89,17 +89,19 @@ class FP8Linear(nn.Linear):
         hp = w.as_subclass(torch.Tensor)
         state = self.scaling["weight"] if self.scaling is not None else None
         if stream is None:
-            w.data = FP8Tensor(hp, dtype=DTypes.FP8E4M3, state=state, with_transpose=True)
+            w.data = FP8Tensor(hp, dtype=DTypes.FP8E4M3, state=state, with_transpose=needs_transposed_copy(*hp.shape))
             self._weight_ready = None
             return
         cur = torch.cuda.current_stream(hp.device)
         stream.wait_stream(cur)
         with torch.cuda.stream(stream):
-            q = FP8Tensor(hp, dtype=DTypes.FP8E4M3, state=state, with_transpose=True)
+            q = FP8Tensor(hp, dtype=DTypes.FP8E4M3, state=state, with_transpose=needs_transposed_copy(*hp.shape))
             ready = torch.cuda.Event()
             ready.record(stream)
         # the new tensors were allocated on `stream` and will be read on the current one
-        for t in (q, q.transposed(), q.fp8_meta.amax):
+        for t in (q, getattr(q, "_transposed", None), q.fp8_meta.amax):
+            if t is None:
+                continue
             t.record_stream(cur)
         w.data = q
         self._weight_ready = ready
@@ -151,9 +153,9 @@ class FP8Linear(nn.Linear):
         hp = w.as_subclass(torch.Tensor)
         with torch.no_grad():
             if weight_scale is not None:
-                w.data = cast_with_scale(hp, weight_scale, DTypes.FP8E4M3, with_transpose=True)
+                w.data = cast_with_scale(hp, weight_scale, DTypes.FP8E4M3, with_transpose=needs_transposed_copy(*hp.shape))
             else:
-                w.data = FP8Tensor(hp, dtype=DTypes.FP8E4M3, with_transpose=True)
+                w.data = FP8Tensor(hp, dtype=DTypes.FP8E4M3, with_transpose=needs_transposed_copy(*hp.shape))
         self._weight_ready = None
 
     def forward(self, input: Union[FP8Tensor, torch.Tensor]) -> torch.Tensor:
@@ -188,7 +190,7 @@ class _FP8Matmul(torch.autograd.Function):
         if type(input) == torch.Tensor:
             x2d = input.reshape(-1, input.shape[-1])
             input = FP8Tensor(x2d, dtype=DTypes.FP8E4M3, state=scaling["input"] if scaling else None,
-                              with_transpose=needs_wgrad)
+                              with_transpose=needs_wgrad and needs_transposed_copy(x2d.shape[0], x2d.shape[1], weight.shape[0]))
         ctx.save_for_backward(input, weight)
         ctx.module = module
         out_dtype = module.out_dtype or torch.float32
