@@ -136,7 +136,8 @@ def _gemm_nt_batch(problems):
     return outs
 
 
-def _operands(mat_a: FP8Tensor, transpose_a: bool, mat_b: FP8Tensor, transpose_b: bool):
+def _operands(mat_a: FP8Tensor, transpose_a: bool, mat_b: FP8Tensor, transpose_b: bool,
+              accumulate_into: Optional[torch.Tensor] = None):
     """(A, B, b_transposed) of the library's D = A . B^T for the reference's D = op_b(B) . op_a(A) (kernel.py:43-44).
 
     Where the reference transposes mat_a (tex.fp8_transpose, kernel.py:43) the library can read it as it is
@@ -148,7 +149,8 @@ def _operands(mat_a: FP8Tensor, transpose_a: bool, mat_b: FP8Tensor, transpose_b
     b_ = mat_b.transposed() if transpose_b else mat_b   # the library's A: always K-contiguous
     if transpose_a:
         return b_, mat_a, False
-    if getattr(mat_a, "_transposed", None) is None and mat_a.dim() == 2 and mat_a.is_contiguous() and \
+    aligned = all(t is None or t.data_ptr() % 16 == 0 for t in (mat_a, b_, accumulate_into))   # 16-byte loads / stores
+    if getattr(mat_a, "_transposed", None) is None and mat_a.dim() == 2 and mat_a.is_contiguous() and aligned and \
             b_transposed_supported(b_.shape[0], mat_a.shape[1], mat_a.shape[0]):
         return b_, mat_a, True
     return b_, mat_a.transposed(), False
@@ -161,8 +163,8 @@ def fp8_matmul_pair(first: dict, second: dict):
     results as two calls; the library lets the two GEMMs share kernel launches."""
     probs = []
     for kw in (first, second):
-        A, B, bt = _operands(kw["mat_a"], kw["transpose_a"], kw["mat_b"], kw["transpose_b"])
         acc = kw.get("accumulate_into")
+        A, B, bt = _operands(kw["mat_a"], kw["transpose_a"], kw["mat_b"], kw["transpose_b"], acc)
         probs.append((A, B, (kw.get("out_dtype") or torch.float32) if acc is None else torch.float32, acc, bt))
     return _gemm_nt_batch(probs)
 
@@ -200,7 +202,7 @@ def fp8_matmul_kernel(
         a_ = mat_a if transpose_a else mat_a.transposed()  # kernel.py:43
         b_ = mat_b.transposed() if transpose_b else mat_b  # kernel.py:44
         return _gemm_nt_fp8(b_, a_, out_dtype, out_state, out_with_transpose)
-    A, B, bt = _operands(mat_a, transpose_a, mat_b, transpose_b)
+    A, B, bt = _operands(mat_a, transpose_a, mat_b, transpose_b, accumulate_into)
     if bt:
         return _gemm_nt_batch([(A, B, out_dtype or torch.float32, accumulate_into, True)])[0]
     return _gemm_nt(A, B, out_dtype or torch.float32, accumulate_into)

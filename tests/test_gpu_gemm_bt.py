@@ -172,3 +172,40 @@ def test_linear_gives_the_same_bits_with_and_without_transposed_copies(master):
     for a, b in zip(*results):
         assert torch.equal(_bits(a), _bits(b))
     assert torch.isfinite(results[0][-4]).all() and results[0][-4].abs().max() > 0   # the accumulated weight gradient
+
+
+def test_operator_falls_back_to_a_transposed_copy_when_the_direct_read_does_not_apply():
+    """fp8_matmul_kernel(mat_a, transpose_a=False, ...) reads mat_a as it is where it can; a misaligned view, a shape
+    with N not a multiple of 16, or a tensor that already carries its transposed copy take the copy.  Same results."""
+    from nanotron_amd.fp8 import FP8Tensor
+    from nanotron_amd.fp8.kernel import _operands, fp8_matmul_kernel
+    from nanotron_amd.fp8.meta import FP8Meta
+
+    one = torch.tensor(1.0)
+    g = torch.Generator().manual_seed(4)
+    K, N, M = 384, 272, 300
+    w = torch.randint(-4, 5, (K, N), generator=g).float()     # mat_a [K, N]: reduced over its rows
+    x = torch.randint(-4, 5, (M, K), generator=g).float()     # mat_b [M, K]
+    want = x @ w
+    X = from_bytes(O.cast_to_fp8(x, one, O.E4M3), 1.0, O.E4M3)
+    W = from_bytes(O.cast_to_fp8(w, one, O.E4M3), 1.0, O.E4M3)
+    assert _operands(W, False, X, False)[2] is True
+    assert torch.equal(fp8_matmul_kernel(W, False, X, False, False).cpu(), want)
+    # misaligned storage
+    buf = torch.empty(K * N + 8, dtype=torch.uint8, device="cuda")
+    view = buf[8:].view(K, N)
+    view.copy_(W.as_subclass(torch.Tensor))
+    Wm = torch.Tensor._make_subclass(FP8Tensor, view)
+    Wm.fp8_meta = FP8Meta(torch.tensor(0.0, device="cuda"), torch.tensor(1.0, device="cuda"), _dt(O.E4M3))
+    assert Wm.data_ptr() % 16 == 8 and _operands(Wm, False, X, False)[2] is False
+    assert torch.equal(fp8_matmul_kernel(Wm, False, X, False, False).cpu(), want)
+    # a tensor that carries its transposed copy uses it
+    W2 = from_bytes(O.cast_to_fp8(w, one, O.E4M3), 1.0, O.E4M3)
+    W2.transposed()
+    assert _operands(W2, False, X, False)[2] is False
+    assert torch.equal(fp8_matmul_kernel(W2, False, X, False, False).cpu(), want)
+    # N not a multiple of 16
+    w3 = torch.randint(-4, 5, (K, 250), generator=g).float()
+    W3 = from_bytes(O.cast_to_fp8(w3, one, O.E4M3), 1.0, O.E4M3)
+    assert _operands(W3, False, X, False)[2] is False
+    assert torch.equal(fp8_matmul_kernel(W3, False, X, False, False).cpu(), x @ w3)
