@@ -384,7 +384,9 @@ void gemm_nt_big_kernel(const BigLaunch L) {
                 // (address-space cast, not a round trip through an integer: the compiler must see that these reads
                 // come from sB, or it waits for every direct-to-LDS load in flight before each of them)
                 int x = bt_x;
-                asm volatile("" : "+v"(x));   // recomputed at every use: eight block offsets kept across the K loop do not fit
+                // half tiles: recomputed at every use, eight block offsets kept across the K loop do not fit their
+                // register budget; whole tiles keep them (1 % faster than recomputing)
+                if constexpr (MI == 4) asm volatile("" : "+v"(x));
                 uint8_t* p = &sB[s][bt_base + ((j << 4) ^ x) + h * (2 * 8 * 256)];
                 const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((tr_ptr)p);
                 const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((tr_ptr)(p + 8 * 256));
