@@ -1,12 +1,13 @@
 // FP8 GEMM for gfx950:  D[M,N] (+)= (A[M,K] . B[N,K]^T) * (1/scale_a)(1/scale_b)
 //
-// Both operands are contiguous along K (the only form the reference issues).  fp32 accumulation on
-// the matrix cores with V_MFMA_F32_32X32X64_F8F6F4 (e4m3 / e5m2 selectable per operand), operand
-// tiles staged in XOR-swizzled LDS, descale + one rounding in the epilogue.
+// Both operands are contiguous along K (the only form the reference issues); the big kernel also takes B as
+// its transpose, a [K, N] tensor.  fp32 accumulation on the matrix cores (e4m3 / e5m2 selectable per
+// operand), operand tiles staged in XOR-swizzled LDS, descale + one rounding in the epilogue to fp32
+// (optionally added to what is there), bf16, fp16 or fp8 bytes.
 //
 // Three kernels:
 //   gemm_nt_big_kernel    (gemm_big.h) 256 x 256 x 128 tiles, 4 waves of 128 x 128 with 16x16x128 MFMAs,
-//                         direct global->LDS buffer loads, two LDS stages, one barrier per K-tile.  The
+//                         loads staged through registers, two LDS stages, one barrier per K-tile.  The
 //                         partial last round of tiles over the CUs is cut into 128-row half tiles.
 //   gemm_nt_kernel        128 x 128 x 128 tiles, 4 waves, loads through registers; small shapes and
 //                         operands beyond the 2 GiB reach of a buffer descriptor's 32-bit offsets.

@@ -18,6 +18,10 @@
 // Global loads: whole tiles (MI = 8) keep one K-tile in flight in registers and write it to LDS a
 // K-tile later, so that every load has a full K-tile of MFMA time to arrive; half tiles (MI = 4) have
 // no registers to spare and load straight into the released LDS stage.
+//
+// Instantiations beside the operand formats and MI: kFp8Out (the outputs are fp8 bytes, cast in the
+// epilogue, with an optional transposed copy and the amax of the results) and kBT (the B operands are
+// given as their transposes, [K, N] tensors, and gathered from LDS with the transposing read).
 #pragma once
 
 namespace ntfp8 {
