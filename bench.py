@@ -35,7 +35,7 @@ PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E peak
 # scaled by what the same counter reads for a 128 MiB copy: x2.0 for FETCH_SIZE, x1.0 for WRITE_SIZE); the figures
 # and the commands are in profiles/hbm_traffic_counters.txt.  Bytes, summed over the GEMM launches of one step /
 # for one launch of the fused quantise kernel on the [4096,4096] bf16 tensor.
-GEMM_TRAFFIC_PER_STEP = {"fetch": 4134.0e6, "write": 1479.7e6}
+GEMM_TRAFFIC_PER_STEP = {"fetch": 4133.3e6, "write": 1478.7e6}
 QUANT_TRAFFIC_PER_LAUNCH = {"fetch": 33.67e6, "write": 16.79e6}
 
 TOKENS = 4096
