@@ -289,3 +289,50 @@ def test_batch_mixes_fp8_and_plain_outputs_and_rejects_bad_requests():
     assert nt.lib.ntfp8_amax_finalize(None, 0, 0, state.data_ptr(), None, 0, amax.data_ptr(), None, st) == codes["a required pointer is NULL"]
     torch.cuda.synchronize()
     assert ctypes.sizeof(nt.GemmDesc) == 112
+
+
+def test_fp8_output_chain_replayed_as_a_graph_matches_eager():
+    """GEMM epilogue atomics into the workspace, the one-wave bookkeeping kernel that zeroes it again and nothing
+    allocated in between: the forward of two chained layers can be captured and replayed; three replays with fresh
+    inputs and unrelated eager work in between, against an eager twin, bit for bit including the scaling state."""
+    from nanotron_amd.fp8 import DTypes, FP8Linear
+
+    def build():
+        torch.manual_seed(5)
+        return (FP8Linear(256, 512, bias=False, device="cuda", out_dtype=DTypes.FP8E4M3, delayed_scaling=True, amax_history_len=4),
+                FP8Linear(512, 256, bias=False, device="cuda", out_dtype=torch.bfloat16, delayed_scaling=True, amax_history_len=4))
+
+    def fwd(layers, x):
+        with torch.no_grad():
+            return layers[1](layers[0](x))
+
+    def inputs(i):
+        return O.normal_tensor(700 + i, (384, 256), 1.0 + 0.2 * i, torch.bfloat16).cuda()
+
+    g_layers, e_layers = build(), build()
+    sx = torch.zeros(384, 256, dtype=torch.bfloat16, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):   # warm-up on the capture stream: every scaling role holds a scale afterwards
+        for i in range(2):
+            sx.copy_(inputs(i))
+            fwd(g_layers, sx)
+    torch.cuda.current_stream().wait_stream(side)
+    for i in range(2):
+        fwd(e_layers, inputs(i))
+    torch.cuda.synchronize()
+    assert g_layers[0].scaling["output"].initialised
+    graph = torch.cuda.CUDAGraph()
+    sx.copy_(inputs(2))
+    with torch.cuda.graph(graph):
+        sy = fwd(g_layers, sx)
+    for i in range(2, 5):
+        x = inputs(i)
+        sx.copy_(x)
+        graph.replay()
+        ye = fwd(e_layers, x)
+        _ = (ye.float() @ ye.float().t()).sum().item()   # unrelated eager work and a synchronisation in between
+        assert torch.equal(sy, ye)
+        for a, b in zip(g_layers, e_layers):
+            for role in a.scaling:
+                assert _same_f32(a.scaling[role]._buf, b.scaling[role]._buf), role
