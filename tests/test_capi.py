@@ -140,3 +140,53 @@ def test_python_api_surface_matches_reference_names():
     from nanotron.fp8.tensor import update_scaling_factor as ref_path_usf  # noqa
 
     assert RefPathLinear is FP8Linear
+
+
+def test_fp8_output_and_transposed_operand_requests_are_validated_before_any_launch():
+    from nanotron_amd import _native as nt
+
+    L = nt.lib
+    P = 0x100000   # fake device pointers, never dereferenced: every call below is refused on the host
+
+    def desc(**kw):
+        d = nt.GemmDesc()
+        d.A, d.scale_a, d.B, d.scale_b, d.D = P, P + (1 << 20), P + (2 << 20), P + (1 << 20) + 64, P + (3 << 20)
+        d.M, d.N, d.K, d.fmt_a, d.fmt_b, d.d_dtype, d.accumulate = 256, 256, 256, 0, 0, 0, 0
+        for k, v in kw.items():
+            setattr(d, k, v)
+        return (nt.GemmDesc * 1)(d)
+
+    assert L.ntfp8_gemm_batch(desc(d_dtype=nt.OUT_E4M3), 1, None) == -1                                 # no scale_d
+    assert L.ntfp8_gemm_batch(desc(d_dtype=nt.OUT_E5M2, scale_d=P + (4 << 20), accumulate=1), 1, None) == -5
+    assert L.ntfp8_gemm_batch(desc(d_dtype=nt.OUT_E4M3, scale_d=P + (4 << 20) + 2), 1, None) == -4        # misaligned scale
+    assert L.ntfp8_gemm_batch(desc(d_dtype=nt.OUT_E4M3, scale_d=P + (4 << 20), D_t=P + (3 << 20) + 64), 1, None) == -7
+    assert L.ntfp8_gemm_batch(desc(d_dtype=nt.OUT_E4M3, scale_d=P + (4 << 20), b_transposed=1), 1, None) == -5
+    assert L.ntfp8_gemm_batch(desc(d_dtype=7), 1, None) == -2
+    assert L.ntfp8_gemm(P, 0, P + (1 << 20), P + (2 << 20), 0, P + (1 << 20), P + (3 << 20), nt.OUT_E4M3, 256, 256, 256, 0, None) == -5
+    # a transposed B operand outside what the kernels serve
+    for m, n, k in [(256, 250, 256), (128, 256, 256), (256, 256, 128), (256, 256, 250)]:
+        assert L.ntfp8_gemm_batch(desc(M=m, N=n, K=k, b_transposed=1), 1, None) == -5, (m, n, k)
+    # amax bookkeeping entry point
+    assert L.ntfp8_amax_finalize(None, 0, 0, P, P + 64, 16, P + 256, None, None) == -1
+    assert L.ntfp8_amax_finalize(P, 5, 0, P + 4096, P + 8192, 16, P + 256, None, None) == -2
+    assert L.ntfp8_amax_finalize(P, 0, 0, P + 4096, P + 8192, 0, P + 256, None, None) == -3     # history without a length
+    assert L.ntfp8_amax_finalize(P, 0, 0, P + 4096, None, 4, P + 256, None, None) == -3           # length without a history
+    assert L.ntfp8_amax_finalize(P, 0, 500, P + 4096, None, 0, P + 256, None, None) == -3
+    assert L.ntfp8_amax_finalize(P, 0, 0, P + 4098, None, 0, P + 256, None, None) == -4
+    assert ctypes.sizeof(nt.GemmDesc) == 112
+
+
+def test_host_policy_for_transposed_copies():
+    import nanotron_amd.fp8.kernel as K
+
+    assert K.b_transposed_supported(4096, 4096, 14336) and K.b_transposed_supported(129, 144, 256)
+    for m, n, k in [(4096, 4090, 4096), (128, 4096, 4096), (4096, 128, 4096), (4096, 4096, 128), (4096, 4096, 4100),
+                    (4096, 1 << 20, 4096)]:
+        assert not K.b_transposed_supported(m, n, k), (m, n, k)
+    # a weight [out, in] is reduced over its rows in dgrad: no copy when in_features qualifies
+    assert not K.needs_transposed_copy(14336, 4096) and K.needs_transposed_copy(14336, 4090) and K.needs_transposed_copy(64, 4096)
+    K.READ_B_TRANSPOSED = False
+    try:
+        assert not K.b_transposed_supported(4096, 4096, 4096) and K.needs_transposed_copy(14336, 4096)
+    finally:
+        K.READ_B_TRANSPOSED = True
