@@ -148,7 +148,9 @@ def gemm_in_step_timing(step, first_index, steps):
         return bracket(lambda: orig_one(a, b, out_dtype, accumulate_into), [(a.shape[0], b.shape[0], a.shape[1])])
 
     def timed_batch(problems):
-        return bracket(lambda: orig_batch(problems), [(p[0].shape[0], p[1].shape[0], p[0].shape[1]) for p in problems])
+        # a fifth element marks a B operand handed over as its [K, N] transpose
+        return bracket(lambda: orig_batch(problems),
+                       [(p[0].shape[0], p[1].shape[1 if len(p) > 4 and p[4] else 0], p[0].shape[1]) for p in problems])
 
     K._gemm_nt, K._gemm_nt_batch = timed_one, timed_batch
     try:
