@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/ntfp8.h"
 
 namespace ntfp8 {
@@ -148,17 +150,17 @@ struct GemmDesc {
 
 __host__ __device__ inline bool is_fp8_out(int d_dtype) { return d_dtype == NTFP8_OUT_E4M3 || d_dtype == NTFP8_OUT_E5M2; }
 
-// compute units of the current device (cached per device)
+// compute units of the current device (cached per device; threads may race to fill an entry, with the same value)
 inline int cu_count() {
-    static int cached[64] = {0};
+    static std::atomic<int> cached[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int v = 0;
+    int v = cached[dev].load(std::memory_order_relaxed);
+    if (v == 0) {
         if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
-        cached[dev] = v;
+        cached[dev].store(v, std::memory_order_relaxed);
     }
-    return cached[dev];
+    return v;
 }
 
 }  // namespace ntfp8
