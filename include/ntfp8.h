@@ -93,6 +93,26 @@ int ntfp8_quantize_delayed(const void* x, int x_dtype, int64_t rows, int64_t col
                            float* amax_out, float* scale_used_out, void* out, void* out_t,
                            void* workspace, void* stream);
 
+/* ntfp8_quantize_delayed for several tensors in one call (each with a zeroed workspace of its own): same results
+ * as the separate calls.  Tensors without a transposed copy that share source type and format share a launch, in
+ * which the reduction and bookkeeping of one tensor run under the streaming of the next instead of in front of a
+ * kernel boundary: the call for the fp8 copies of all weights after an optimizer step (the reference has no
+ * counterpart: it quantises a weight once, src/nanotron/fp8/parameter.py:27). */
+#define NTFP8_MAX_BATCH 64   /* problems / tensors per batched call */
+typedef struct ntfp8_quant_desc {
+    const void* x;
+    int x_dtype, fmt, margin, history_len;
+    int64_t rows, cols;
+    float* scale_state;
+    float* amax_history;
+    float* amax_out;
+    float* scale_used_out;   /* may be NULL */
+    void* out;
+    void* out_t;             /* may be NULL */
+    void* workspace;
+} ntfp8_quant_desc;
+int ntfp8_quantize_delayed_batch(const ntfp8_quant_desc* tensors, int count, void* stream);
+
 /* out = out_dtype(fp32(fp8) * (1 / *scale)).  Replaces tex.cast_from_fp8
  * (src/nanotron/fp8/tensor.py:74) with meta.inverse_scale (src/nanotron/fp8/meta.py:36-37). */
 int ntfp8_cast_from_fp8(const void* in, int fmt, const float* scale, int64_t n, void* out, int out_dtype,
@@ -137,7 +157,6 @@ typedef struct ntfp8_gemm_desc {
      * and outputs other than fp8; anything else returns NTFP8_ERR_UNSUPPORTED (transpose B and pass 0). */
     int b_transposed;
 } ntfp8_gemm_desc;
-#define NTFP8_MAX_BATCH 64
 int ntfp8_gemm_batch(const ntfp8_gemm_desc* problems, int count, void* stream);
 
 /* fp8 GEMM output ("return an fp8 tensor as output", the TODO at src/nanotron/fp8/linear.py:63-64):

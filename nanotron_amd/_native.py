@@ -40,6 +40,14 @@ class GemmDesc(ctypes.Structure):
                 ("scale_d", _vp), ("D_t", _vp), ("amax_workspace", _vp), ("b_transposed", _i)]
 
 
+class QuantDesc(ctypes.Structure):
+    """`ntfp8_quant_desc` of include/ntfp8.h."""
+    _fields_ = [("x", _vp), ("x_dtype", _i), ("fmt", _i), ("margin", _i), ("history_len", _i),
+                ("rows", _i64), ("cols", _i64),
+                ("scale_state", _vp), ("amax_history", _vp), ("amax_out", _vp), ("scale_used_out", _vp),
+                ("out", _vp), ("out_t", _vp), ("workspace", _vp)]
+
+
 SIGNATURES = {
     "ntfp8_version": (_i, []),
     "ntfp8_strerror": (_c.c_char_p, [_i]),
@@ -49,6 +57,7 @@ SIGNATURES = {
     "ntfp8_cast_to_fp8": (_i, [_vp, _i, _i64, _i64, _vp, _i, _vp, _vp, _vp]),
     "ntfp8_quantize_current": (_i, [_vp, _i, _i64, _i64, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp]),
     "ntfp8_quantize_delayed": (_i, [_vp, _i, _i64, _i64, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "ntfp8_quantize_delayed_batch": (_i, [_c.POINTER(QuantDesc), _i, _vp]),
     "ntfp8_cast_from_fp8": (_i, [_vp, _i, _vp, _i64, _vp, _i, _vp]),
     "ntfp8_transpose": (_i, [_vp, _i64, _i64, _vp, _vp]),
     "ntfp8_gemm": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i64, _i64, _i64, _i, _vp]),
@@ -101,6 +110,21 @@ def workspace_and_stream(device: torch.device) -> Tuple[torch.Tensor, int]:
         ws = torch.zeros(WORKSPACE_BYTES // 4, dtype=torch.int32, device=device)
         _workspaces[(idx, st)] = ws
     return ws, st
+
+
+_pools: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def workspace_pool(device: torch.device, count: int) -> Tuple[torch.Tensor, int]:
+    """([>= count, WORKSPACE_BYTES / 4] zero-initialised workspaces, stream pointer) for torch's current stream on
+    `device`: one workspace per tensor of a batched call (kernels leave them zero)."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    st = stream_ptr(device)
+    pool = _pools.get((idx, st))
+    if pool is None or pool.shape[0] < count:
+        pool = torch.zeros(max(count, 16), WORKSPACE_BYTES // 4, dtype=torch.int32, device=device)
+        _pools[(idx, st)] = pool
+    return pool, st
 
 
 def workspace(device: torch.device) -> torch.Tensor:

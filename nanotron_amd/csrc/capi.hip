@@ -11,6 +11,7 @@ int run_transpose(const void* in, int64_t rows, int64_t cols, void* out, hipStre
 int run_update_scale(const float* amax, const float* old_scale, int fmt, int margin, float* out, int64_t n,
                      hipStream_t st);
 int run_amax_finalize(Workspace* ws, const ScalarIO& io, hipStream_t st);
+int run_quant_delayed_batch(const QuantDesc* q, int count, hipStream_t st);
 int run_gemm(const GemmDesc& g, hipStream_t st);
 int run_gemm_batch(const GemmDesc* g, int n, hipStream_t st);
 
@@ -196,6 +197,34 @@ int ntfp8_quantize_delayed(const void* x, int x_dtype, int64_t rows, int64_t col
     ScalarIO io = {nullptr, amax_out, scale_used_out, scale_state, amax_history, history_len, fmt, margin};
     return run_quant(kModeDelayed, x, x_dtype, rows, cols, fmt, static_cast<uint8_t*>(out), static_cast<uint8_t*>(out_t),
                      scale_state, static_cast<Workspace*>(workspace), io, static_cast<hipStream_t>(stream));
+}
+
+int ntfp8_quantize_delayed_batch(const ntfp8_quant_desc* tensors, int count, void* stream) {
+    if (!tensors) return NTFP8_ERR_NULL;
+    if (count <= 0 || count > NTFP8_MAX_BATCH) return NTFP8_ERR_SIZE;
+    QuantDesc q[NTFP8_MAX_BATCH];
+    for (int i = 0; i < count; ++i) {
+        const ntfp8_quant_desc& t = tensors[i];
+        int64_t n;
+        if (!t.scale_state || !t.amax_history || !t.amax_out || !t.workspace || (!t.out && !t.out_t)) return NTFP8_ERR_NULL;
+        int rc = check_quant_common(t.x, t.x_dtype, t.rows, t.cols, t.fmt, t.margin, &n);
+        if (rc) return rc;
+        if (t.history_len < 1 || t.history_len > kMaxHistory) return NTFP8_ERR_SIZE;
+        if (!is_aligned(t.scale_state, 4) || !is_aligned(t.amax_history, 4) || !is_aligned(t.amax_out, 4) ||
+            !is_aligned(t.workspace, 4) || (t.scale_used_out && !is_aligned(t.scale_used_out, 4)))
+            return NTFP8_ERR_ALIGN;
+        rc = check_outputs(t.x, t.x_dtype, n, t.out, t.out_t);
+        if (rc) return rc;
+        for (int j = 0; j < i; ++j)   // the tensors run concurrently: nothing one of them writes may be shared
+            if (tensors[j].workspace == t.workspace || tensors[j].scale_state == t.scale_state ||
+                tensors[j].amax_history == t.amax_history || tensors[j].amax_out == t.amax_out ||
+                (t.out && tensors[j].out == t.out) || (t.out_t && tensors[j].out_t == t.out_t))
+                return NTFP8_ERR_ALIAS;
+        q[i] = QuantDesc{t.x, t.x_dtype, t.rows, t.cols, t.fmt, t.out, t.out_t, t.workspace,
+                         ScalarIO{nullptr, t.amax_out, t.scale_used_out, t.scale_state, t.amax_history, t.history_len, t.fmt,
+                                  t.margin}};
+    }
+    return run_quant_delayed_batch(q, count, static_cast<hipStream_t>(stream));
 }
 
 int ntfp8_cast_from_fp8(const void* in, int fmt, const float* scale, int64_t n, void* out, int out_dtype, void* stream) {

@@ -47,6 +47,18 @@ struct ScalarIO {
     int margin;
 };
 
+// one tensor of a batched quantise call as the launchers see it (validated by the C entry point)
+struct QuantDesc {
+    const void* x;
+    int x_dtype;
+    int64_t rows, cols;
+    int fmt;
+    void* out;
+    void* out_t;
+    void* ws;
+    ScalarIO io;
+};
+
 template <int F>
 struct Fmt;
 template <>

@@ -208,9 +208,12 @@ __device__ inline void finalize_wave(Workspace* ws, const ScalarIO& io, int mode
     }
 }
 
+// `bid` of `nblocks`: this workgroup's place among the workgroups that reduce the same tensor (the whole grid,
+// except in a launch that carries several tensors).
 template <int THREADS>
 __device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, const ScalarIO& io, int mode,
-                                            const EpiloguePrefetch& pre) {
+                                            const EpiloguePrefetch& pre, uint32_t bid = blockIdx.x,
+                                            uint32_t nblocks = gridDim.x) {
     __shared__ uint32_t s_part[THREADS / 64];
     __shared__ bool s_last;
     const uint32_t wm = wave_max_u32(m_f32bits);
@@ -223,14 +226,14 @@ __device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, c
         // Two-level arrival count: a block publishes into the slot of its group and draws a ticket there; the
         // last block of a group draws a ticket of the launch.  All blocks finish at about the same time, and
         // their atomics on one address would queue one behind the other.
-        const uint32_t grp = blockIdx.x % kMaxSlots;
+        const uint32_t grp = bid % kMaxSlots;
         const uint32_t old = __hip_atomic_fetch_max(&ws->slot[grp].bits, bm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         asm volatile("s_waitcnt vmcnt(0)" ::"v"(old) : "memory");   // the max is in place before the ticket is drawn
-        const uint32_t in_group = (gridDim.x - grp + kMaxSlots - 1) / kMaxSlots;
+        const uint32_t in_group = (nblocks - grp + kMaxSlots - 1) / kMaxSlots;
         const uint32_t t = __hip_atomic_fetch_add(&ws->slot[grp].ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         bool last = false;
         if (t == in_group - 1) {
-            const uint32_t groups = gridDim.x < (uint32_t)kMaxSlots ? gridDim.x : (uint32_t)kMaxSlots;
+            const uint32_t groups = nblocks < (uint32_t)kMaxSlots ? nblocks : (uint32_t)kMaxSlots;
             const uint32_t t2 = __hip_atomic_fetch_add(&ws->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             last = (t2 == groups - 1);
         }
@@ -256,10 +259,9 @@ __device__ __forceinline__ bool degenerate_scale(float s) {
 // ---------------------------------------------------------------------------------------------
 // Flat (no transpose) kernel: amax only, cast only, or both (delayed scaling).
 template <typename S, int F, int MODE>
-__global__ __launch_bounds__(kFlatThreads) void quant_flat_kernel(const typename ElemOf<S>::type* __restrict__ x,
-                                                              int64_t n_vec, int64_t n, uint8_t* __restrict__ out,
-                                                              const float* __restrict__ scale_ptr, Workspace* ws,
-                                                              ScalarIO io) {
+__device__ __forceinline__ void quant_flat_body(const typename ElemOf<S>::type* __restrict__ x, int64_t n_vec, int64_t n,
+                                                uint8_t* __restrict__ out, const float* __restrict__ scale_ptr,
+                                                Workspace* ws, const ScalarIO& io, uint32_t bid, uint32_t nblocks) {
     typedef Src<S> L;
     constexpr bool kCast = MODE != kModeAmaxOnly;
     constexpr bool kAmax = MODE != kModeCastOnly;
@@ -272,8 +274,8 @@ __global__ __launch_bounds__(kFlatThreads) void quant_flat_kernel(const typename
     EpiloguePrefetch pre = {0.0f, 1.0f};
     if constexpr (kAmax) pre = prefetch_epilogue(io, MODE);
     uint32_t m_run = 0;  // in source-format bits
-    const int64_t stride = (int64_t)gridDim.x * kFlatThreads;
-    int64_t i = (int64_t)blockIdx.x * kFlatThreads + threadIdx.x;
+    const int64_t stride = (int64_t)nblocks * kFlatThreads;
+    int64_t i = (int64_t)bid * kFlatThreads + threadIdx.x;
     // two groups per trip: four (bf16) or eight (fp32) 128-bit loads in flight per lane
     for (; i + stride < n_vec; i += 2 * stride) {
         float v0[16], v1[16];
@@ -302,13 +304,48 @@ __global__ __launch_bounds__(kFlatThreads) void quant_flat_kernel(const typename
         }
     }
     // elements the vector body does not cover (tail, or everything when a pointer is misaligned)
-    for (int64_t j = n_vec * kVec + (int64_t)blockIdx.x * kFlatThreads + threadIdx.x; j < n; j += stride) {
+    for (int64_t j = n_vec * kVec + (int64_t)bid * kFlatThreads + threadIdx.x; j < n; j += stride) {
         uint32_t m;
         const float xv = L::load1(x + j, m);
         if constexpr (kAmax) m_run = m > m_run ? m : m_run;
         if constexpr (kCast) out[j] = encode1<F>(xv, scale);
     }
-    if constexpr (kAmax) publish_and_finalize<kFlatThreads>(L::to_f32_bits(m_run), ws, io, MODE, pre);
+    if constexpr (kAmax) publish_and_finalize<kFlatThreads>(L::to_f32_bits(m_run), ws, io, MODE, pre, bid, nblocks);
+}
+
+template <typename S, int F, int MODE>
+__global__ __launch_bounds__(kFlatThreads) void quant_flat_kernel(const typename ElemOf<S>::type* __restrict__ x,
+                                                              int64_t n_vec, int64_t n, uint8_t* __restrict__ out,
+                                                              const float* __restrict__ scale_ptr, Workspace* ws,
+                                                              ScalarIO io) {
+    quant_flat_body<S, F, MODE>(x, n_vec, n, out, scale_ptr, ws, io, blockIdx.x, gridDim.x);
+}
+
+// Several tensors, one launch (the fused delayed-scaling step of each): the workgroups of tensor t follow those of
+// tensor t - 1, so the tail of one tensor (its last loads, its reduction, its bookkeeping) runs under the streaming
+// of the next instead of in front of a kernel boundary.  Every tensor has its own workspace.
+constexpr int kMaxMulti = 16;
+struct MultiQuant {
+    struct Tensor {
+        const void* x;
+        uint8_t* out;
+        int64_t n_vec, n;
+        Workspace* ws;
+        ScalarIO io;
+        int first_block, blocks;
+    } t[kMaxMulti];
+    int count;
+};
+
+template <typename S, int F>
+__global__ __launch_bounds__(kFlatThreads) void quant_flat_multi_kernel(const MultiQuant Q) {
+    int which = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxMulti; ++i)
+        if (i < Q.count && (int)blockIdx.x >= Q.t[i].first_block) which = i;
+    const MultiQuant::Tensor& T = Q.t[which];
+    quant_flat_body<S, F, kModeDelayed>(static_cast<const typename ElemOf<S>::type*>(T.x), T.n_vec, T.n, T.out,
+                                        T.io.scale_state, T.ws, T.io, blockIdx.x - T.first_block, T.blocks);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -542,6 +579,68 @@ int run_quant(int mode, const void* x, int x_dtype, int64_t rows, int64_t cols, 
         case NTFP8_F16: return dispatch_fmt_flat<f16_tag>(fmt, mode, x, n, vec_ok, out, scale_ptr, ws, io, st);
         default: return dispatch_fmt_flat<bf16_tag>(fmt, mode, x, n, vec_ok, out, scale_ptr, ws, io, st);
     }
+}
+
+template <typename S, int F>
+static int launch_flat_multi(const QuantDesc* const* q, int count, hipStream_t st) {
+    MultiQuant Q = {};
+    Q.count = count;
+    int blocks = 0;
+    for (int i = 0; i < count; ++i) {
+        const QuantDesc& d = *q[i];
+        const int64_t n = d.rows * d.cols;
+        const bool vec_ok = aligned(d.x, 16) && aligned(d.out, 16);
+        MultiQuant::Tensor& T = Q.t[i];
+        T.x = d.x;
+        T.out = static_cast<uint8_t*>(d.out);
+        T.n = n;
+        T.n_vec = vec_ok ? n / kVec : 0;
+        T.ws = static_cast<Workspace*>(d.ws);
+        T.io = d.io;
+        T.first_block = blocks;
+        T.blocks = grid_for(T.n_vec > 0 ? (T.n_vec + 1) / 2 : n, kFlatThreads, 1);
+        blocks += T.blocks;
+    }
+    hipLaunchKernelGGL((quant_flat_multi_kernel<S, F>), dim3(blocks), dim3(kFlatThreads), 0, st, Q);
+    return check_launch();
+}
+
+template <typename S>
+static int dispatch_flat_multi(int fmt, const QuantDesc* const* q, int count, hipStream_t st) {
+    return fmt == kE4M3 ? launch_flat_multi<S, kE4M3>(q, count, st) : launch_flat_multi<S, kE5M2>(q, count, st);
+}
+
+// The fused delayed-scaling step of several tensors.  Tensors without a transposed copy that share source type and
+// format go out together, up to kMaxMulti per launch; the others one by one.
+int run_quant_delayed_batch(const QuantDesc* q, int count, hipStream_t st) {
+    bool done[NTFP8_MAX_BATCH] = {false};
+    for (int i = 0; i < count; ++i) {
+        if (done[i]) continue;
+        done[i] = true;
+        if (q[i].out_t != nullptr || q[i].out == nullptr) {
+            const int rc = run_quant(kModeDelayed, q[i].x, q[i].x_dtype, q[i].rows, q[i].cols, q[i].fmt,
+                                     static_cast<uint8_t*>(q[i].out), static_cast<uint8_t*>(q[i].out_t), q[i].io.scale_state,
+                                     static_cast<Workspace*>(q[i].ws), q[i].io, st);
+            if (rc != NTFP8_OK) return rc;
+            continue;
+        }
+        const QuantDesc* group[kMaxMulti];
+        int cnt = 0;
+        group[cnt++] = &q[i];
+        for (int j = i + 1; j < count && cnt < kMaxMulti; ++j)
+            if (!done[j] && q[j].out_t == nullptr && q[j].out != nullptr && q[j].x_dtype == q[i].x_dtype && q[j].fmt == q[i].fmt) {
+                group[cnt++] = &q[j];
+                done[j] = true;
+            }
+        int rc;
+        switch (q[i].x_dtype) {
+            case NTFP8_F32: rc = dispatch_flat_multi<float>(q[i].fmt, group, cnt, st); break;
+            case NTFP8_F16: rc = dispatch_flat_multi<f16_tag>(q[i].fmt, group, cnt, st); break;
+            default: rc = dispatch_flat_multi<bf16_tag>(q[i].fmt, group, cnt, st); break;
+        }
+        if (rc != NTFP8_OK) return rc;
+    }
+    return NTFP8_OK;
 }
 
 int run_dequant(const void* in, int fmt, const float* scale, int64_t n, void* out, int out_dtype, hipStream_t st) {

@@ -346,3 +346,79 @@ def test_convert_tensor_to_fp8_with_given_meta():
     meta = FP8Meta(torch.tensor(8.0, device="cuda"), torch.tensor(32.0, device="cuda"), DTypes.FP8E5M2)
     got = convert_tensor_to_fp8(x.cuda(), meta).cpu()
     assert torch.equal(got, O.cast_to_fp8(x, torch.tensor(32.0), O.E5M2))
+
+
+def test_batched_delayed_quantise_equals_the_separate_calls():
+    """ntfp8_quantize_delayed_batch: tensors of one source type without a transposed copy share a launch, the rest go
+    out one by one; bytes, transposed bytes, amax, scale used, next scale and history equal the separate calls."""
+    from nanotron_amd.fp8 import DelayedScaling, DTypes, FP8Tensor
+    from nanotron_amd.fp8.tensor import quantize_delayed_batch
+
+    shapes = [(512, 384), (1000, 37), (128, 256), (4096, 1024), (3, 5), (256, 128), (777,), (2048, 2048)]
+    dtypes = [torch.bfloat16, torch.bfloat16, torch.float32, torch.bfloat16, torch.float16, torch.bfloat16, torch.float32,
+              torch.bfloat16]
+    with_t = [False, False, False, False, False, True, False, True]
+    tensors, states, twins = [], [], []
+    for i, (shape, dt) in enumerate(zip(shapes, dtypes)):
+        x = O.normal_tensor(900 + i, shape, 0.3 * (i + 1), dt)
+        if i == 3:
+            x[17, 5] = float("nan")   # a NaN tensor: NaN amax, scale held
+        tensors.append(x.cuda())
+        st = DelayedScaling(DTypes.FP8E4M3, history_len=4 + i, device="cuda")
+        st._buf[0] = float(2.0 ** (i - 2))
+        st._buf[1:3] = torch.tensor([0.5 * i, 3.0])
+        st.initialised = True
+        tw = DelayedScaling(DTypes.FP8E4M3, history_len=4 + i, device="cuda")
+        tw._buf.copy_(st._buf)
+        tw.initialised = True
+        states.append(st)
+        twins.append(tw)
+    for step in range(2):   # the second step runs on the scales the first one left
+        got = quantize_delayed_batch(tensors, DTypes.FP8E4M3, states, with_t)
+        for x, q, st, tw, wt in zip(tensors, got, states, twins, with_t):
+            want = FP8Tensor(x, DTypes.FP8E4M3, state=tw, with_transpose=wt)
+            assert q.shape == x.shape
+            assert torch.equal(q.as_subclass(torch.Tensor), want.as_subclass(torch.Tensor))
+            if wt:
+                assert torch.equal(q.transposed().as_subclass(torch.Tensor), want.transposed().as_subclass(torch.Tensor))
+            for a, b in ((q.fp8_meta.amax, want.fp8_meta.amax), (q.fp8_meta.scale, want.fp8_meta.scale), (st._buf, tw._buf)):
+                a, b = a.float().cpu().reshape(-1), b.float().cpu().reshape(-1)
+                assert bool(torch.all((a.view(torch.int32) == b.view(torch.int32)) | (a.isnan() & b.isnan())))
+    from nanotron_amd import _native as nt
+
+    pool, _ = nt.workspace_pool(torch.device("cuda", 0), 1)
+    assert int(pool.abs().sum().item()) == 0, "every workspace of the pool is left zeroed"
+
+
+def test_requantize_fp8_weights_batches_and_matches_per_layer_refresh():
+    from torch import nn
+
+    from nanotron_amd.fp8 import FP8Linear
+    from nanotron_amd.fp8.optim import requantize_fp8_weights
+
+    def build():
+        torch.manual_seed(3)
+        return nn.Sequential(FP8Linear(256, 512, bias=False, device="cuda", delayed_scaling=True, amax_history_len=4),
+                             FP8Linear(512, 250, bias=False, device="cuda", delayed_scaling=True, amax_history_len=4),
+                             FP8Linear(250, 64, bias=True, device="cuda", delayed_scaling=True, amax_history_len=4),
+                             FP8Linear(64, 64, bias=False, device="cuda"))   # no delayed scaling: refreshed on its own
+    a, b = build(), build()
+    for step in range(3):   # step 0: no weight role holds a scale yet; steps 1, 2: one batched call
+        with torch.no_grad():
+            for m in (a, b):
+                for p in m.parameters():
+                    p.as_subclass(torch.Tensor).mul_(1.0 + 0.25 * (step + 1))
+        assert requantize_fp8_weights(a) == 4
+        for lin in b:
+            lin.requantize_weight()
+        for la, lb in zip(a, b):
+            assert torch.equal(la.weight.data.as_subclass(torch.Tensor), lb.weight.data.as_subclass(torch.Tensor))
+            ta, tb = getattr(la.weight.data, "_transposed", None), getattr(lb.weight.data, "_transposed", None)
+            assert (ta is None) == (tb is None)
+            if ta is not None:
+                assert torch.equal(ta.as_subclass(torch.Tensor), tb.as_subclass(torch.Tensor))
+            assert torch.equal(la.weight.fp8_meta.scale, lb.weight.fp8_meta.scale)
+            if la.scaling is not None:
+                assert torch.equal(la.scaling["weight"]._buf, lb.scaling["weight"]._buf)
+    x = torch.randn(300, 256, device="cuda")
+    assert torch.equal(a(x), b(x))
