@@ -190,3 +190,35 @@ def test_host_policy_for_transposed_copies():
         assert not K.b_transposed_supported(4096, 4096, 4096) and K.needs_transposed_copy(14336, 4096)
     finally:
         K.READ_B_TRANSPOSED = True
+
+
+def test_batched_quantise_requests_are_validated_before_any_launch():
+    from nanotron_amd import _native as nt
+
+    L = nt.lib
+    P = 0x200000
+
+    def desc(k, **kw):
+        d = nt.QuantDesc()
+        base = P + k * (1 << 20)
+        d.x, d.x_dtype, d.fmt, d.margin, d.history_len, d.rows, d.cols = base, 2, 0, 0, 16, 4, 4
+        d.scale_state, d.amax_history, d.amax_out, d.out, d.workspace = base + 4096, base + 4100, base + 8192, base + 12288, base + 16384
+        for name, v in kw.items():
+            setattr(d, name, v)
+        return d
+
+    one = lambda d: (nt.QuantDesc * 1)(d)
+    assert L.ntfp8_quantize_delayed_batch(None, 1, None) == -1
+    assert L.ntfp8_quantize_delayed_batch(one(desc(0)), 0, None) == -3
+    assert L.ntfp8_quantize_delayed_batch(one(desc(0)), 65, None) == -3
+    assert L.ntfp8_quantize_delayed_batch(one(desc(0, workspace=None)), 1, None) == -1
+    assert L.ntfp8_quantize_delayed_batch(one(desc(0, out=None)), 1, None) == -1
+    assert L.ntfp8_quantize_delayed_batch(one(desc(0, x_dtype=9)), 1, None) == -2
+    assert L.ntfp8_quantize_delayed_batch(one(desc(0, history_len=0)), 1, None) == -3
+    assert L.ntfp8_quantize_delayed_batch(one(desc(0, rows=0)), 1, None) == -3
+    assert L.ntfp8_quantize_delayed_batch(one(desc(0, scale_state=P + 4098)), 1, None) == -4
+    assert L.ntfp8_quantize_delayed_batch(one(desc(0, out=P + 8)), 1, None) == -7            # output over the input
+    shared = (nt.QuantDesc * 2)(desc(0), desc(1, workspace=P + 16384))                         # two tensors, one workspace
+    assert L.ntfp8_quantize_delayed_batch(shared, 2, None) == -7
+    shared = (nt.QuantDesc * 2)(desc(0), desc(1, scale_state=P + 4096))                        # ... or one scaling state
+    assert L.ntfp8_quantize_delayed_batch(shared, 2, None) == -7
