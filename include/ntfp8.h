@@ -15,7 +15,11 @@
  *   - 2-D operands are row-major and contiguous; fp8 bytes are OCP e4m3fn / e5m2;
  *   - `workspace` is NTFP8_WORKSPACE_BYTES of device memory that must be zero before its first
  *     use; kernels leave it zero again, so it can be reused by stream-ordered calls.  Calls
- *     that may overlap (different streams) need distinct workspaces.
+ *     that may overlap (different streams) need distinct workspaces;
+ *   - every scale argument is the SCALE (x_fp8 = x * scale) unless an entry point or descriptor field says
+ *     that it takes the inverse scale, the form Transformer Engine's functions are handed by the reference
+ *     (`meta.inverse_scale`, src/nanotron/fp8/meta.py:36-37).  For the power-of-two scales this path produces
+ *     (src/nanotron/fp8/tensor.py:97-103) both forms give the same bits: 1 / (1 / s) == s exactly.
  */
 #ifndef NTFP8_H
 #define NTFP8_H
@@ -27,7 +31,7 @@
 extern "C" {
 #endif
 
-#define NTFP8_VERSION 1
+#define NTFP8_VERSION 2
 #define NTFP8_WORKSPACE_BYTES 2048
 
 /* FP8 storage formats.  Reference: DTypes.FP8E4M3 / DTypes.FP8E5M2 (src/nanotron/fp8/dtypes.py:4-7),
@@ -75,6 +79,15 @@ float ntfp8_update_scaling_factor_host(float amax, float old_scale, int fmt, int
 int ntfp8_cast_to_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* scale,
                       int fmt, void* out, void* out_t, void* stream);
 
+/* tex.cast_to_fp8(input, scale, amax, scale_inv, otype) with all of its effects (src/nanotron/fp8/tensor.py:65; the
+ * arithmetic lives in Transformer Engine, which the reference does not vendor: the effects below are its published
+ * behaviour): out = saturating_rne_fp8(fp32(x) * *scale); *amax_inout = max(*amax_inout, max|x|) (a NaN on either
+ * side is kept; Transformer Engine's own maximum drops NaN inputs, an un-pinned corner); *scale_inv_out = 1 / *scale.
+ * amax_inout and scale_inv_out may each be NULL; with both NULL this is ntfp8_cast_to_fp8 without a transposed
+ * copy and needs no workspace. */
+int ntfp8_te_cast_to_fp8(const void* x, int x_dtype, int64_t n, const float* scale, float* amax_inout,
+                         float* scale_inv_out, int fmt, void* out, void* workspace, void* stream);
+
 /* FP8Tensor.__new__ in one call (src/nanotron/fp8/tensor.py:25-28): current scaling.
  * amax pass, scale from amax starting at 1.0, cast pass.  If amax_history is not NULL the
  * delayed-scaling state is updated as well (history rolled, *scale_state = next scale), which
@@ -92,6 +105,16 @@ int ntfp8_quantize_delayed(const void* x, int x_dtype, int64_t rows, int64_t col
                            float* scale_state, float* amax_history, int history_len,
                            float* amax_out, float* scale_used_out, void* out, void* out_t,
                            void* workspace, void* stream);
+
+/* One delayed-scaling step of TWO roles that quantise the same tensor, e4m3 and e5m2, in a single pass over x
+ * (4 bytes of traffic per bf16 element instead of 2 x 3; no counterpart in the reference).  Results equal, bit for
+ * bit, ntfp8_quantize_delayed called once per format: the amax is shared, each role keeps its own scale and
+ * history.  scale_used_out_* may be NULL. */
+int ntfp8_quantize_delayed_dual(const void* x, int x_dtype, int64_t n, int margin,
+                                float* scale_state_e4m3, float* amax_history_e4m3,
+                                float* scale_state_e5m2, float* amax_history_e5m2, int history_len,
+                                float* amax_out, float* scale_used_out_e4m3, float* scale_used_out_e5m2,
+                                void* out_e4m3, void* out_e5m2, void* workspace, void* stream);
 
 /* ntfp8_quantize_delayed for several tensors in one call (each with a zeroed workspace of its own): same results
  * as the separate calls.  Tensors without a transposed copy that share source type and format share a launch, in
@@ -113,10 +136,15 @@ typedef struct ntfp8_quant_desc {
 } ntfp8_quant_desc;
 int ntfp8_quantize_delayed_batch(const ntfp8_quant_desc* tensors, int count, void* stream);
 
+
 /* out = out_dtype(fp32(fp8) * (1 / *scale)).  Replaces tex.cast_from_fp8
  * (src/nanotron/fp8/tensor.py:74) with meta.inverse_scale (src/nanotron/fp8/meta.py:36-37). */
 int ntfp8_cast_from_fp8(const void* in, int fmt, const float* scale, int64_t n, void* out, int out_dtype,
                         void* stream);
+/* The same with the inverse scale as argument, which is what tex.cast_from_fp8 receives at
+ * src/nanotron/fp8/tensor.py:74: out = out_dtype(fp32(fp8) * *scale_inv). */
+int ntfp8_cast_from_fp8_scale_inv(const void* in, int fmt, const float* scale_inv, int64_t n, void* out, int out_dtype,
+                                  void* stream);
 
 /* Byte transpose [rows, cols] -> [cols, rows].  Replaces tex.fp8_transpose
  * (src/nanotron/fp8/kernel.py:43-44). */
@@ -156,7 +184,20 @@ typedef struct ntfp8_gemm_desc {
      * tensor as it is.  Served for N a multiple of 16, M and N above 128, K at least 256, operands below 2 GiB
      * and outputs other than fp8; anything else returns NTFP8_ERR_UNSUPPORTED (transpose B and pass 0). */
     int b_transposed;
+    /* NULL, or bias[N] of type bias_dtype (NTFP8_F32 / NTFP8_F16 / NTFP8_BF16), added to the descaled fp32 result
+     * before the single rounding to d_dtype: D = round(fp32(acc * descale) + bias[n]).  This is the `bias` /
+     * `bias_type` pair of tex.te_gemm, which the reference leaves empty (src/nanotron/fp8/kernel.py:29-32) and adds
+     * outside instead (src/nanotron/fp8/linear.py:62,65).  For an fp32 output the result equals the separate
+     * addition bit for bit; for 16-bit and fp8 outputs it saves the intermediate rounding.  Not together with
+     * b_transposed (NTFP8_ERR_UNSUPPORTED): the backward GEMMs that use it have no bias. */
+    const void* bias;
+    int bias_dtype;
+    /* != 0: scale_a and scale_b point to INVERSE scales, the form tex.te_gemm is handed
+     * (meta.inverse_scale, src/nanotron/fp8/kernel.py:48,52): the sum is multiplied by them, not divided. */
+    int scales_are_inverse;
 } ntfp8_gemm_desc;
+/* A call that returns an error has launched nothing: every problem is validated, and matched to a kernel, before
+ * the first launch. */
 int ntfp8_gemm_batch(const ntfp8_gemm_desc* problems, int count, void* stream);
 
 /* fp8 GEMM output ("return an fp8 tensor as output", the TODO at src/nanotron/fp8/linear.py:63-64):

@@ -37,7 +37,8 @@ class GemmDesc(ctypes.Structure):
     _fields_ = [("A", _vp), ("scale_a", _vp), ("B", _vp), ("scale_b", _vp), ("D", _vp),
                 ("M", _i64), ("N", _i64), ("K", _i64),
                 ("fmt_a", _i), ("fmt_b", _i), ("d_dtype", _i), ("accumulate", _i),
-                ("scale_d", _vp), ("D_t", _vp), ("amax_workspace", _vp), ("b_transposed", _i)]
+                ("scale_d", _vp), ("D_t", _vp), ("amax_workspace", _vp), ("b_transposed", _i),
+                ("bias", _vp), ("bias_dtype", _i), ("scales_are_inverse", _i)]
 
 
 class QuantDesc(ctypes.Structure):
@@ -58,7 +59,10 @@ SIGNATURES = {
     "ntfp8_quantize_current": (_i, [_vp, _i, _i64, _i64, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp]),
     "ntfp8_quantize_delayed": (_i, [_vp, _i, _i64, _i64, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "ntfp8_quantize_delayed_batch": (_i, [_c.POINTER(QuantDesc), _i, _vp]),
+    "ntfp8_quantize_delayed_dual": (_i, [_vp, _i, _i64, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "ntfp8_te_cast_to_fp8": (_i, [_vp, _i, _i64, _vp, _vp, _vp, _i, _vp, _vp, _vp]),
     "ntfp8_cast_from_fp8": (_i, [_vp, _i, _vp, _i64, _vp, _i, _vp]),
+    "ntfp8_cast_from_fp8_scale_inv": (_i, [_vp, _i, _vp, _i64, _vp, _i, _vp]),
     "ntfp8_transpose": (_i, [_vp, _i64, _i64, _vp, _vp]),
     "ntfp8_gemm": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i64, _i64, _i64, _i, _vp]),
     "ntfp8_gemm_batch": (_i, [_c.POINTER(GemmDesc), _i, _vp]),

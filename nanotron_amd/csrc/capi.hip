@@ -6,7 +6,11 @@ namespace ntfp8 {
 
 int run_quant(int mode, const void* x, int x_dtype, int64_t rows, int64_t cols, int fmt, uint8_t* out, uint8_t* out_t,
               const float* scale_ptr, Workspace* ws, const ScalarIO& io, hipStream_t st);
-int run_dequant(const void* in, int fmt, const float* scale, int64_t n, void* out, int out_dtype, hipStream_t st);
+int run_dequant(const void* in, int fmt, const float* scale, int is_inverse, int64_t n, void* out, int out_dtype,
+                hipStream_t st);
+int run_quant_dual(const void* x, int x_dtype, int64_t n, uint8_t* out_e4m3, uint8_t* out_e5m2, Workspace* ws,
+                   const ScalarIO& io_e4m3, const ScalarIO& io_e5m2, hipStream_t st);
+
 int run_transpose(const void* in, int64_t rows, int64_t cols, void* out, hipStream_t st);
 int run_update_scale(const float* amax, const float* old_scale, int fmt, int margin, float* out, int64_t n,
                      hipStream_t st);
@@ -73,8 +77,15 @@ int check_gemm(const ntfp8_gemm_desc& p, GemmDesc* g) {
         return NTFP8_ERR_ALIGN;
     const size_t db = (size_t)mn * dtype_size(p.d_dtype);
     if (overlap(p.A, (size_t)mk, p.D, db) || overlap(p.B, (size_t)nk, p.D, db)) return NTFP8_ERR_ALIAS;
+    if (p.bias) {
+        if (p.b_transposed) return NTFP8_ERR_UNSUPPORTED;
+        if (!dtype_ok(p.bias_dtype)) return NTFP8_ERR_ENUM;
+        if (!is_aligned(p.bias, dtype_size(p.bias_dtype))) return NTFP8_ERR_ALIGN;
+        if (overlap(p.bias, (size_t)N * dtype_size(p.bias_dtype), p.D, db)) return NTFP8_ERR_ALIAS;
+    }
     *g = GemmDesc{p.A, p.fmt_a, p.scale_a, p.B, p.fmt_b, p.scale_b, p.D, p.d_dtype, (int)M, (int)N, (int)K, p.accumulate ? 1 : 0,
-                  nullptr, nullptr, nullptr, p.b_transposed ? 1 : 0};
+                  nullptr, nullptr, nullptr, p.b_transposed ? 1 : 0, p.bias, p.bias ? p.bias_dtype : NTFP8_F32,
+                  p.scales_are_inverse ? 1 : 0};
     if (p.b_transposed && fp8_out) return NTFP8_ERR_UNSUPPORTED;
     if (fp8_out) {
         if (!is_aligned(p.scale_d, 4) || (p.amax_workspace && !is_aligned(p.amax_workspace, 4))) return NTFP8_ERR_ALIGN;
@@ -199,32 +210,91 @@ int ntfp8_quantize_delayed(const void* x, int x_dtype, int64_t rows, int64_t col
                      scale_state, static_cast<Workspace*>(workspace), io, static_cast<hipStream_t>(stream));
 }
 
-int ntfp8_quantize_delayed_batch(const ntfp8_quant_desc* tensors, int count, void* stream) {
+// validation of a batched quantise call; fills q[0 .. count)
+static int check_quant_batch(const ntfp8_quant_desc* tensors, int count, int max_count, bool own_workspaces, QuantDesc* q) {
     if (!tensors) return NTFP8_ERR_NULL;
-    if (count <= 0 || count > NTFP8_MAX_BATCH) return NTFP8_ERR_SIZE;
-    QuantDesc q[NTFP8_MAX_BATCH];
+    if (count <= 0 || count > max_count) return NTFP8_ERR_SIZE;
     for (int i = 0; i < count; ++i) {
         const ntfp8_quant_desc& t = tensors[i];
         int64_t n;
-        if (!t.scale_state || !t.amax_history || !t.amax_out || !t.workspace || (!t.out && !t.out_t)) return NTFP8_ERR_NULL;
+        if (!t.scale_state || !t.amax_history || !t.amax_out || (own_workspaces && !t.workspace) || (!t.out && !t.out_t))
+            return NTFP8_ERR_NULL;
         int rc = check_quant_common(t.x, t.x_dtype, t.rows, t.cols, t.fmt, t.margin, &n);
         if (rc) return rc;
         if (t.history_len < 1 || t.history_len > kMaxHistory) return NTFP8_ERR_SIZE;
         if (!is_aligned(t.scale_state, 4) || !is_aligned(t.amax_history, 4) || !is_aligned(t.amax_out, 4) ||
-            !is_aligned(t.workspace, 4) || (t.scale_used_out && !is_aligned(t.scale_used_out, 4)))
+            (own_workspaces && !is_aligned(t.workspace, 4)) || (t.scale_used_out && !is_aligned(t.scale_used_out, 4)))
             return NTFP8_ERR_ALIGN;
         rc = check_outputs(t.x, t.x_dtype, n, t.out, t.out_t);
         if (rc) return rc;
         for (int j = 0; j < i; ++j)   // the tensors run concurrently: nothing one of them writes may be shared
-            if (tensors[j].workspace == t.workspace || tensors[j].scale_state == t.scale_state ||
+            if ((own_workspaces && tensors[j].workspace == t.workspace) || tensors[j].scale_state == t.scale_state ||
                 tensors[j].amax_history == t.amax_history || tensors[j].amax_out == t.amax_out ||
                 (t.out && tensors[j].out == t.out) || (t.out_t && tensors[j].out_t == t.out_t))
                 return NTFP8_ERR_ALIAS;
-        q[i] = QuantDesc{t.x, t.x_dtype, t.rows, t.cols, t.fmt, t.out, t.out_t, t.workspace,
+        q[i] = QuantDesc{t.x, t.x_dtype, t.rows, t.cols, t.fmt, t.out, t.out_t, own_workspaces ? t.workspace : nullptr,
                          ScalarIO{nullptr, t.amax_out, t.scale_used_out, t.scale_state, t.amax_history, t.history_len, t.fmt,
                                   t.margin}};
     }
+    return NTFP8_OK;
+}
+
+int ntfp8_quantize_delayed_batch(const ntfp8_quant_desc* tensors, int count, void* stream) {
+    QuantDesc q[NTFP8_MAX_BATCH];
+    const int rc = check_quant_batch(tensors, count, NTFP8_MAX_BATCH, true, q);
+    if (rc) return rc;
     return run_quant_delayed_batch(q, count, static_cast<hipStream_t>(stream));
+}
+
+int ntfp8_te_cast_to_fp8(const void* x, int x_dtype, int64_t n, const float* scale, float* amax_inout, float* scale_inv_out,
+                         int fmt, void* out, void* workspace, void* stream) {
+    int64_t nn;
+    if (!scale || !out) return NTFP8_ERR_NULL;
+    const bool bookkeeping = amax_inout || scale_inv_out;
+    if (bookkeeping && !workspace) return NTFP8_ERR_NULL;
+    int rc = check_quant_common(x, x_dtype, n, 1, fmt, 0, &nn);
+    if (rc) return rc;
+    if (!is_aligned(scale, 4) || (amax_inout && !is_aligned(amax_inout, 4)) || (scale_inv_out && !is_aligned(scale_inv_out, 4)) ||
+        (workspace && !is_aligned(workspace, 4)))
+        return NTFP8_ERR_ALIGN;
+    rc = check_outputs(x, x_dtype, nn, out, nullptr);
+    if (rc) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (!bookkeeping) {
+        ScalarIO io = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, fmt, 0};
+        return run_quant(kModeCastOnly, x, x_dtype, nn, 1, fmt, static_cast<uint8_t*>(out), nullptr, scale, nullptr, io, st);
+    }
+    // the fused pass: cast with *scale, amax of x, no history
+    ScalarIO io = {nullptr, amax_inout, nullptr, const_cast<float*>(scale), nullptr, 0, fmt, 0, amax_inout, scale_inv_out};
+    rc = run_quant(kModeDelayed, x, x_dtype, nn, 1, fmt, static_cast<uint8_t*>(out), nullptr, scale,
+                   static_cast<Workspace*>(workspace), io, st);
+    return rc;
+}
+
+int ntfp8_quantize_delayed_dual(const void* x, int x_dtype, int64_t n, int margin, float* scale_state_e4m3,
+                                float* amax_history_e4m3, float* scale_state_e5m2, float* amax_history_e5m2, int history_len,
+                                float* amax_out, float* scale_used_out_e4m3, float* scale_used_out_e5m2, void* out_e4m3,
+                                void* out_e5m2, void* workspace, void* stream) {
+    int64_t nn;
+    if (!scale_state_e4m3 || !amax_history_e4m3 || !scale_state_e5m2 || !amax_history_e5m2 || !amax_out || !out_e4m3 ||
+        !out_e5m2 || !workspace)
+        return NTFP8_ERR_NULL;
+    int rc = check_quant_common(x, x_dtype, n, 1, NTFP8_E4M3, margin, &nn);
+    if (rc) return rc;
+    if (history_len < 1 || history_len > kMaxHistory) return NTFP8_ERR_SIZE;
+    if (!is_aligned(scale_state_e4m3, 4) || !is_aligned(amax_history_e4m3, 4) || !is_aligned(scale_state_e5m2, 4) ||
+        !is_aligned(amax_history_e5m2, 4) || !is_aligned(amax_out, 4) || !is_aligned(workspace, 4) ||
+        (scale_used_out_e4m3 && !is_aligned(scale_used_out_e4m3, 4)) || (scale_used_out_e5m2 && !is_aligned(scale_used_out_e5m2, 4)))
+        return NTFP8_ERR_ALIGN;
+    rc = check_outputs(x, x_dtype, nn, out_e4m3, out_e5m2);
+    if (rc) return rc;
+    if (scale_state_e4m3 == scale_state_e5m2 || amax_history_e4m3 == amax_history_e5m2 ||
+        (scale_used_out_e4m3 && scale_used_out_e4m3 == scale_used_out_e5m2))
+        return NTFP8_ERR_ALIAS;
+    ScalarIO io0 = {nullptr, amax_out, scale_used_out_e4m3, scale_state_e4m3, amax_history_e4m3, history_len, NTFP8_E4M3, margin};
+    ScalarIO io1 = {nullptr, amax_out, scale_used_out_e5m2, scale_state_e5m2, amax_history_e5m2, history_len, NTFP8_E5M2, margin};
+    return run_quant_dual(x, x_dtype, nn, static_cast<uint8_t*>(out_e4m3), static_cast<uint8_t*>(out_e5m2),
+                          static_cast<Workspace*>(workspace), io0, io1, static_cast<hipStream_t>(stream));
 }
 
 int ntfp8_cast_from_fp8(const void* in, int fmt, const float* scale, int64_t n, void* out, int out_dtype, void* stream) {
@@ -233,7 +303,17 @@ int ntfp8_cast_from_fp8(const void* in, int fmt, const float* scale, int64_t n, 
     if (n <= 0 || n > (1LL << 46)) return NTFP8_ERR_SIZE;
     if (!is_aligned(scale, 4) || !is_aligned(out, dtype_size(out_dtype))) return NTFP8_ERR_ALIGN;
     if (overlap(in, (size_t)n, out, (size_t)n * dtype_size(out_dtype))) return NTFP8_ERR_ALIAS;
-    return run_dequant(in, fmt, scale, n, out, out_dtype, static_cast<hipStream_t>(stream));
+    return run_dequant(in, fmt, scale, 0, n, out, out_dtype, static_cast<hipStream_t>(stream));
+}
+
+int ntfp8_cast_from_fp8_scale_inv(const void* in, int fmt, const float* scale_inv, int64_t n, void* out, int out_dtype,
+                                  void* stream) {
+    if (!in || !scale_inv || !out) return NTFP8_ERR_NULL;
+    if (!fmt_ok(fmt) || !dtype_ok(out_dtype)) return NTFP8_ERR_ENUM;
+    if (n <= 0 || n > (1LL << 46)) return NTFP8_ERR_SIZE;
+    if (!is_aligned(scale_inv, 4) || !is_aligned(out, dtype_size(out_dtype))) return NTFP8_ERR_ALIGN;
+    if (overlap(in, (size_t)n, out, (size_t)n * dtype_size(out_dtype))) return NTFP8_ERR_ALIAS;
+    return run_dequant(in, fmt, scale_inv, 1, n, out, out_dtype, static_cast<hipStream_t>(stream));
 }
 
 int ntfp8_transpose(const void* in, int64_t rows, int64_t cols, void* out, void* stream) {
@@ -247,7 +327,8 @@ int ntfp8_transpose(const void* in, int64_t rows, int64_t cols, void* out, void*
 int ntfp8_gemm(const void* A, int fmt_a, const float* scale_a, const void* B, int fmt_b, const float* scale_b, void* D,
                int d_dtype, int64_t M, int64_t N, int64_t K, int accumulate, void* stream) {
     if (is_fp8_out(d_dtype)) return NTFP8_ERR_UNSUPPORTED;   // fp8 outputs carry more arguments: ntfp8_gemm_batch
-    const ntfp8_gemm_desc p = {A, scale_a, B, scale_b, D, M, N, K, fmt_a, fmt_b, d_dtype, accumulate, nullptr, nullptr, nullptr, 0};
+    const ntfp8_gemm_desc p = {A, scale_a, B, scale_b, D, M, N, K, fmt_a, fmt_b, d_dtype, accumulate, nullptr, nullptr, nullptr, 0,
+                               nullptr, NTFP8_F32, 0};
     GemmDesc g;
     const int rc = check_gemm(p, &g);
     if (rc) return rc;

@@ -45,6 +45,9 @@ struct ScalarIO {
     int hist_len;
     int fmt;
     int margin;
+    // Transformer-Engine-shaped cast (tex.cast_to_fp8 takes `amax` and `scale_inv` tensors and updates both):
+    const float* amax_in;    // not NULL: *amax_out = max(*amax_in, amax of this tensor), NaN from either side kept
+    float* scale_inv_out;    // not NULL: receives 1 / (scale the bytes were produced with)
 };
 
 // one tensor of a batched quantise call as the launchers see it (validated by the C entry point)
@@ -158,6 +161,10 @@ struct GemmDesc {
     void* Dt;
     void* ws;
     int tb;   // B is given as [K, N] row-major (its transpose)
+    // optional bias[N] added to the descaled fp32 result before the single rounding (NULL: none)
+    const void* bias;
+    int bias_dtype;
+    int scale_inv;   // scale_a / scale_b point to inverse scales (what tex.te_gemm receives): multiplied, not divided by
 };
 
 __host__ __device__ inline bool is_fp8_out(int d_dtype) { return d_dtype == NTFP8_OUT_E4M3 || d_dtype == NTFP8_OUT_E5M2; }

@@ -26,7 +26,7 @@ template <int FA, int FB, int DT, bool kAcc>
 __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                                void* __restrict__ Dv, const float* __restrict__ scale_a,
                                                                const float* __restrict__ scale_b, int M, int N, int K,
-                                                               int tiles_m, int tiles_n, Fp8Out fp8) {
+                                                               int tiles_m, int tiles_n, Fp8Out fp8, GemmExtras ex) {
     __shared__ __attribute__((aligned(16))) uint8_t sA[kBM * kBK];
     __shared__ __attribute__((aligned(16))) uint8_t sB[kBN * kBK];
 
@@ -106,7 +106,11 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(const uint8_t* __
         }
     }
 
-    const float alpha = (1.0f / *scale_a) * (1.0f / *scale_b);
+    float alpha = descale_factor(scale_a, scale_b, ex.scale_inv);
+    if (ex.bias) {   // uniform
+        add_bias32<2, 2>(acc, alpha, ex.bias, ex.bias_dtype, N, n0 + wn, lane);
+        alpha = 1.0f;
+    }
     if constexpr (DT == NTFP8_OUT_E4M3 || DT == NTFP8_OUT_E5M2) {
         constexpr int F = DT == NTFP8_OUT_E4M3 ? kE4M3 : kE5M2;
         const float scale_d = *fp8.scale;
@@ -123,7 +127,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nt_kernel(const uint8_t* __
 template <int FA, int FB, int DT, bool kAcc>
 __global__ void gemm_nt_naive_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, void* __restrict__ Dv,
                                      const float* __restrict__ scale_a, const float* __restrict__ scale_b, int M, int N,
-                                     int K, Fp8Out fp8) {
+                                     int K, Fp8Out fp8, GemmExtras ex) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const bool live = idx < (int64_t)M * N;
     if (!live && !(DT == NTFP8_OUT_E4M3 || DT == NTFP8_OUT_E5M2)) return;
@@ -136,7 +140,8 @@ __global__ void gemm_nt_naive_kernel(const uint8_t* __restrict__ A, const uint8_
                                     : __builtin_amdgcn_cvt_f32_bf8((int)B[(int64_t)n * K + k], 0);
         acc += a * b;
     }
-    float v = acc * ((1.0f / *scale_a) * (1.0f / *scale_b));
+    float v = acc * descale_factor(scale_a, scale_b, ex.scale_inv);
+    if (ex.bias && live) v = v + bias_at(ex.bias, ex.bias_dtype, n);
     if constexpr (DT == NTFP8_OUT_E4M3 || DT == NTFP8_OUT_E5M2) {
         // whole waves get here (the amax reduction runs over all 64 lanes); lanes past the end hold zeros
         constexpr int F = DT == NTFP8_OUT_E4M3 ? kE4M3 : kE5M2;
@@ -213,12 +218,14 @@ static int launch_big(const GemmDesc* const* g, int n, hipStream_t st) {
         p.d_dtype = d.d_dtype;
         p.accumulate = d.accumulate;
         p.fp8 = Fp8Out{d.sd, static_cast<uint8_t*>(d.Dt), static_cast<Workspace*>(d.ws)};
+        p.ex = GemmExtras{d.bias, d.bias_dtype, d.scale_inv};
         tiles += p.tiles_m * p.tiles_n;
     }
     const int rem = tiles % cu_count();
     L.tail_tiles = (rem != 0 && 2 * rem <= cu_count()) ? rem : 0;
     L.full_blocks = tiles - L.tail_tiles;
     L.round_size = cu_count();
+    (void)hipGetLastError();   // an error left behind by an unrelated earlier call is not this launch's
     if (L.full_blocks > 0)
         hipLaunchKernelGGL((gemm_nt_big_kernel<FA, FB, 8, kFp8Out, kBT>), dim3(L.full_blocks), dim3(kBigThreads), 0, st, L);
     if (L.tail_tiles > 0)
@@ -231,14 +238,16 @@ static int launch_small(const GemmDesc& g, int path, hipStream_t st) {
     const uint8_t* a = static_cast<const uint8_t*>(g.A);
     const uint8_t* b = static_cast<const uint8_t*>(g.B);
     const Fp8Out fp8 = {g.sd, static_cast<uint8_t*>(g.Dt), static_cast<Workspace*>(g.ws)};
+    const GemmExtras ex = {g.bias, g.bias_dtype, g.scale_inv};
+    (void)hipGetLastError();   // an error left behind by an unrelated earlier call is not this launch's
     if (path == kPathSmall) {
         const int tm = (g.M + kBM - 1) / kBM, tn = (g.N + kBN - 1) / kBN;
         hipLaunchKernelGGL((gemm_nt_kernel<FA, FB, DT, kAcc>), dim3(tm * tn), dim3(kGemmThreads), 0, st, a, b, g.D, g.sa,
-                           g.sb, g.M, g.N, g.K, tm, tn, fp8);
+                           g.sb, g.M, g.N, g.K, tm, tn, fp8, ex);
     } else {
         const int64_t blocks = ((int64_t)g.M * g.N + 255) / 256;
         hipLaunchKernelGGL((gemm_nt_naive_kernel<FA, FB, DT, kAcc>), dim3((int)blocks), dim3(256), 0, st, a, b, g.D, g.sa,
-                           g.sb, g.M, g.N, g.K, fp8);
+                           g.sb, g.M, g.N, g.K, fp8, ex);
     }
     return hipGetLastError() == hipSuccess ? NTFP8_OK : NTFP8_ERR_LAUNCH;
 }
@@ -276,6 +285,9 @@ int run_gemm(const GemmDesc& g, hipStream_t st) {
 int run_gemm_batch(const GemmDesc* g, int n, hipStream_t st) {
     bool done[64] = {false};
     if (n > 64) return NTFP8_ERR_SIZE;
+    // a problem no kernel serves fails the whole call before anything is launched
+    for (int i = 0; i < n; ++i)
+        if (path_of(g[i]) == kPathNone) return NTFP8_ERR_UNSUPPORTED;
     for (int i = 0; i < n; ++i) {
         if (done[i]) continue;
         const GemmDesc* group[kBigMaxProblems];

@@ -57,12 +57,18 @@ __device__ __forceinline__ void sched_fence() { __builtin_amdgcn_sched_barrier(0
 
 // Epilogue of one wave: MI x NJ accumulator blocks of 16 x 16, block (i, j) at rows m_base + 16 i,
 // columns n_base + 16 j.  Descale, optional fp32 accumulate, one rounding, store.
-template <int DT, bool kAcc, int MI, int NJ>
+// kBias: bv[j][e] = bias of column n_base + 16 j + 4 (lane / 16) + e, added to the descaled value before the rounding.
+template <int DT, bool kAcc, int MI, int NJ, bool kBias = false>
 __device__ __forceinline__ void store_wave_tile16(const v4f (&acc)[MI][NJ], void* __restrict__ Dv, float alpha, int M,
-                                                  int N, int m_base, int n_base, int lane) {
+                                                  int N, int m_base, int n_base, int lane, const float (*bv)[4] = nullptr) {
     typedef typename OutT<DT>::type O;
     O* D = static_cast<O*>(Dv);
     const int mrow = lane & 15, q = lane >> 4;
+    // element e of block (i, j): descaled, plus bias if there is one (two separately rounded fp32 operations)
+    auto val = [&](int i, int j, int e) -> float {
+        if constexpr (kBias) return acc[i][j][e] * alpha + bv[j][e];
+        else return acc[i][j][e] * alpha;
+    };
     if constexpr (DT != NTFP8_F32) {
         // 16-bit outputs: a lane's 4 consecutive n are only 8 bytes.  Exchanging registers of two
         // neighbouring blocks between lane rows gives every lane 8 consecutive n (16 bytes) of one
@@ -74,10 +80,10 @@ __device__ __forceinline__ void store_wave_tile16(const v4f (&acc)[MI][NJ], void
                 const int m = m_base + i * 16 + mrow;
 #pragma unroll
                 for (int j = 0; j < NJ; j += 2) {
-                    uint32_t x0 = OutT<DT>::pack2(acc[i][j][0] * alpha, acc[i][j][1] * alpha);
-                    uint32_t x1 = OutT<DT>::pack2(acc[i][j][2] * alpha, acc[i][j][3] * alpha);
-                    uint32_t y0 = OutT<DT>::pack2(acc[i][j + 1][0] * alpha, acc[i][j + 1][1] * alpha);
-                    uint32_t y1 = OutT<DT>::pack2(acc[i][j + 1][2] * alpha, acc[i][j + 1][3] * alpha);
+                    uint32_t x0 = OutT<DT>::pack2(val(i, j, 0), val(i, j, 1));
+                    uint32_t x1 = OutT<DT>::pack2(val(i, j, 2), val(i, j, 3));
+                    uint32_t y0 = OutT<DT>::pack2(val(i, j + 1, 0), val(i, j + 1, 1));
+                    uint32_t y1 = OutT<DT>::pack2(val(i, j + 1, 2), val(i, j + 1, 3));
                     swap_rows16(x0, y0);
                     swap_rows16(x1, y1);
                     // lane row q now holds n 8 (q / 2) .. + 7 of block j + (q & 1): x = first four, y = last four
@@ -113,7 +119,7 @@ __device__ __forceinline__ void store_wave_tile16(const v4f (&acc)[MI][NJ], void
             O* dp = D + (int64_t)m * N + n;
             float v[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = acc[i][j][e] * alpha;
+            for (int e = 0; e < 4; ++e) v[e] = val(i, j, e);
             if (vec_ok && n + 3 < N) {
                 if constexpr (DT == NTFP8_F32) {
                     v4f o = {v[0], v[1], v[2], v[3]};
@@ -158,10 +164,15 @@ __device__ __forceinline__ void reg_store4(__amdgpu_buffer_rsrc_t r, uint32_t vo
 // All stores go through buffer descriptors of M N bytes: rows past the end fall outside and are dropped, columns
 // past the end get an offset that does; nothing is predicated, which keeps the scalar registers of the epilogue
 // (and with them the register budget of the K loop before it) small.
-template <int F, int MI, int NJ>
+template <int F, int MI, int NJ, bool kBias = false>
 __device__ __forceinline__ uint32_t store_wave_tile16_fp8(const v4f (&acc)[MI][NJ], uint8_t* __restrict__ D,
                                                           uint8_t* __restrict__ Dt, float alpha, float scale_d, bool slow,
-                                                          int M, int N, int m_base, int n_base, int lane) {
+                                                          int M, int N, int m_base, int n_base, int lane,
+                                                          const float (*bv)[4] = nullptr) {
+    auto val = [&](int i, int j, int e) -> float {
+        if constexpr (kBias) return acc[i][j][e] * alpha + bv[j][e];
+        else return acc[i][j][e] * alpha;
+    };
     static_assert(NJ % 4 == 0, "blocks are exchanged four at a time");
     const int mrow = lane & 15, q = lane >> 4;
     uint32_t amax = 0;
@@ -176,8 +187,7 @@ __device__ __forceinline__ uint32_t store_wave_tile16_fp8(const v4f (&acc)[MI][N
         uint32_t w[NJ];
 #pragma unroll
         for (int j = 0; j < NJ; ++j)
-            w[j] = quant4<F>(acc[i][j][0] * alpha, acc[i][j][1] * alpha, acc[i][j][2] * alpha, acc[i][j][3] * alpha, scale_d,
-                             slow, amax);
+            w[j] = quant4<F>(val(i, j, 0), val(i, j, 1), val(i, j, 2), val(i, j, 3), scale_d, slow, amax);
         if (Dt) {   // uniform
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
@@ -222,6 +232,7 @@ struct BigProblem {
     int d_dtype;            // NTFP8_F32 / NTFP8_F16 / NTFP8_BF16 / NTFP8_OUT_E4M3 / NTFP8_OUT_E5M2
     int accumulate;         // fp32 outputs only: D += result
     Fp8Out fp8;             // fp8 outputs only
+    GemmExtras ex;          // bias, inverse-scale flag
 };
 constexpr int kBigMaxProblems = 4;
 struct BigLaunch {
@@ -310,7 +321,7 @@ void gemm_nt_big_kernel(const BigLaunch L) {
     const int ld_kc = ((lane & 7) ^ (lane >> 3) ^ (wave & 1)) << 4;
     // chunks of the last K-tile at k >= K must read as zero, not as the start of the next row
     const bool tail_dead = (KT - 1) * kBK + ld_kc >= K;
-    const float alpha = (1.0f / *P.scale_a) * (1.0f / *P.scale_b);
+    const float alpha = descale_factor(P.scale_a, P.scale_b, P.ex.scale_inv);
 
     {
         constexpr int LA = MI * 2 * 16 / 8 / kBigWaves;  // wave-level loads of the A tile per wave per stage
@@ -619,25 +630,39 @@ void gemm_nt_big_kernel(const BigLaunch L) {
         back(No{}, No{}, f);
         }
 
-        // output type and accumulation are properties of the problem, not of the kernel (fp8 outputs apart)
-        if constexpr (kFp8Out) {
-            const float scale_d = *P.fp8.scale;
-            const bool slow = scale_is_degenerate(scale_d);
-            const uint32_t amax =
-                P.d_dtype == NTFP8_OUT_E4M3
-                    ? store_wave_tile16_fp8<kE4M3, MI, kBigNJ>(acc, static_cast<uint8_t*>(Dv), P.fp8.Dt, alpha, scale_d, slow, M,
-                                                               N, m0 + wm, n0 + wn, lane)
-                    : store_wave_tile16_fp8<kE5M2, MI, kBigNJ>(acc, static_cast<uint8_t*>(Dv), P.fp8.Dt, alpha, scale_d, slow, M,
-                                                               N, m0 + wm, n0 + wn, lane);
-            publish_amax(amax, P.fp8.ws);
-        } else if (P.d_dtype == NTFP8_BF16) {
-            store_wave_tile16<NTFP8_BF16, false, MI, kBigNJ>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
-        } else if (P.d_dtype == NTFP8_F16) {
-            store_wave_tile16<NTFP8_F16, false, MI, kBigNJ>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
-        } else if (P.accumulate) {
-            store_wave_tile16<NTFP8_F32, true, MI, kBigNJ>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
+        // output type, accumulation and bias are properties of the problem, not of the kernel (fp8 outputs apart)
+        auto epilogue = [&](auto bias_tag, const float (*bv)[4]) {
+            constexpr bool kBias = decltype(bias_tag)::value;
+            if constexpr (kFp8Out) {
+                const float scale_d = *P.fp8.scale;
+                const bool slow = scale_is_degenerate(scale_d);
+                const uint32_t amax =
+                    P.d_dtype == NTFP8_OUT_E4M3
+                        ? store_wave_tile16_fp8<kE4M3, MI, kBigNJ, kBias>(acc, static_cast<uint8_t*>(Dv), P.fp8.Dt, alpha, scale_d,
+                                                                          slow, M, N, m0 + wm, n0 + wn, lane, bv)
+                        : store_wave_tile16_fp8<kE5M2, MI, kBigNJ, kBias>(acc, static_cast<uint8_t*>(Dv), P.fp8.Dt, alpha, scale_d,
+                                                                          slow, M, N, m0 + wm, n0 + wn, lane, bv);
+                publish_amax(amax, P.fp8.ws);
+            } else if (P.d_dtype == NTFP8_BF16) {
+                store_wave_tile16<NTFP8_BF16, false, MI, kBigNJ, kBias>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane, bv);
+            } else if (P.d_dtype == NTFP8_F16) {
+                store_wave_tile16<NTFP8_F16, false, MI, kBigNJ, kBias>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane, bv);
+            } else if (P.accumulate) {
+                store_wave_tile16<NTFP8_F32, true, MI, kBigNJ, kBias>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane, bv);
+            } else {
+                store_wave_tile16<NTFP8_F32, false, MI, kBigNJ, kBias>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane, bv);
+            }
+        };
+        // (no bias together with a transposed B operand: the backward GEMMs that read one have none, and their
+        // instantiation has no registers to spare for the second set of epilogues)
+        bool with_bias = false;
+        if constexpr (!kBT) with_bias = P.ex.bias != nullptr;   // uniform
+        if (with_bias) {
+            float bv[kBigNJ][4];
+            load_bias16<kBigNJ>(bv, P.ex.bias, P.ex.bias_dtype, N, n0 + wn, lane);
+            epilogue(std::true_type{}, bv);
         } else {
-            store_wave_tile16<NTFP8_F32, false, MI, kBigNJ>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane);
+            epilogue(std::false_type{}, nullptr);
         }
     }
 }

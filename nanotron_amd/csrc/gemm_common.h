@@ -96,6 +96,64 @@ __device__ __forceinline__ v16f mfma_32x32x64(v8i b_frag, v8i a_frag, v16f c) {
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b_frag, a_frag, c, FB, FA, 0, 0, 0, 0);
 }
 
+// scale product applied to the accumulated sum: the operands' scales divide it; inverse scales (the form
+// tex.te_gemm is handed, src/nanotron/fp8/kernel.py:48,52) multiply it
+__device__ __forceinline__ float descale_factor(const float* scale_a, const float* scale_b, int scale_inv) {
+    const float sa = *scale_a, sb = *scale_b;
+    return scale_inv ? sa * sb : (1.0f / sa) * (1.0f / sb);
+}
+
+// element n of a bias vector of any supported type, as fp32 (exact)
+__device__ __forceinline__ float bias_at(const void* bias, int dtype, int n) {
+    if (dtype == NTFP8_F32) return static_cast<const float*>(bias)[n];
+    const uint32_t h = static_cast<const uint16_t*>(bias)[n];
+    return dtype == NTFP8_BF16 ? bf16_bits_to_float(h) : half_bits_to_float(h);
+}
+
+// Bias in the epilogue: D = round(fp32(acc * alpha) + bias[n]), two separately rounded fp32 operations before the
+// single rounding to the output type (what `output + bias` does to an fp32 GEMM output, src/nanotron/fp8/linear.py:65).
+// load_bias16: the bias values of the columns a lane owns in 16 x 16 accumulator blocks, bv[j][e] = bias of column
+// n_base + 16 j + 4 (lane / 16) + e (zero past N: those columns are never stored).
+template <int NJ>
+__device__ __forceinline__ void load_bias16(float (&bv)[NJ][4], const void* bias, int bias_dtype, int N, int n_base, int lane) {
+    const int q = lane >> 4;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int n = n_base + j * 16 + q * 4 + e;
+            bv[j][e] = n < N ? bias_at(bias, bias_dtype, n) : 0.0f;
+        }
+}
+// 32 x 32 accumulator blocks (the small kernel, off the fast path): acc <- fp32(acc * alpha) + bias[n] in place, after
+// which the store routines run unchanged with alpha = 1 (a multiplication by one changes nothing).
+template <int MI, int NJ>
+__device__ __forceinline__ void add_bias32(v16f (&acc)[MI][NJ], float alpha, const void* bias, int bias_dtype, int N,
+                                           int n_base, int lane) {
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float b[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int n = n_base + j * 32 + g * 8 + (lane >> 5) * 4 + e;
+                b[e] = n < N ? bias_at(bias, bias_dtype, n) : 0.0f;
+            }
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[i][j][g * 4 + e] = acc[i][j][g * 4 + e] * alpha + b[e];
+        }
+}
+
+// what a problem carries beside its operands and output
+struct GemmExtras {
+    const void* bias;   // NULL, or bias[N]
+    int bias_dtype;     // NTFP8_F32 / NTFP8_F16 / NTFP8_BF16
+    int scale_inv;      // the scale pointers hold inverse scales
+};
+
 // tile order: XCD-contiguous, then kGroupM row-tiles swept before moving along N
 __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int& pid_m, int& pid_n) {
     int pid = blockIdx.x;

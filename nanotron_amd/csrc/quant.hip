@@ -160,12 +160,20 @@ __device__ __forceinline__ EpiloguePrefetch prefetch_epilogue(const ScalarIO& io
 // Bookkeeping of one launch, run by one wave (lanes 0..63 of a workgroup) once every workgroup's maximum is in
 // the slots: amax, history roll, next scale; leaves the workspace zeroed.  Every global access is one round
 // trip for the whole wave instead of one per history entry.
-__device__ inline void finalize_wave(Workspace* ws, const ScalarIO& io, int mode, const EpiloguePrefetch& pre) {
+//
+// collect_amax: the maximum over the slots as a bit pattern (NaN patterns normalised to the quiet NaN).
+__device__ inline uint32_t collect_amax(Workspace* ws) {
     const int lane = threadIdx.x;
     uint32_t bits = 0;
     if (lane < kMaxSlots) bits = __hip_atomic_load(&ws->slot[lane].bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     bits = wave_max_u32(bits);
     if (bits > kInfBits) bits = kNanBits;
+    return bits;
+}
+
+// bookkeep: what one tensor role learns from the amax `bits` of this launch.
+__device__ inline void bookkeep(uint32_t bits, const ScalarIO& io, int mode, const EpiloguePrefetch& pre) {
+    const int lane = threadIdx.x;
     const float a = __uint_as_float(bits);
     float used;
     if (mode == kModeAmaxOnly) {
@@ -197,15 +205,35 @@ __device__ inline void finalize_wave(Workspace* ws, const ScalarIO& io, int mode
         if (hm > kInfBits) hm = kNanBits;
     }
     if (lane == 0) {
-        *io.amax_out = a;
+        uint32_t out_bits = bits;
+        if (io.amax_in) {   // running maximum kept by the caller (NaN patterns compare above everything)
+            uint32_t prev = __float_as_uint(*io.amax_in) & 0x7fffffffu;
+            if (prev > kInfBits) prev = kNanBits;
+            out_bits = prev > out_bits ? prev : out_bits;
+        }
+        if (io.amax_out) *io.amax_out = __uint_as_float(out_bits);
         if (io.scale_out) *io.scale_out = used;
+        if (io.scale_inv_out) *io.scale_inv_out = 1.0f / used;
         if (io.hist) *io.scale_state = update_scale(__uint_as_float(hm), used, io.fmt, io.margin);
-        __hip_atomic_store(&ws->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+}
+
+__device__ inline void clear_workspace(Workspace* ws) {
+    const int lane = threadIdx.x;
+    if (lane == 0) __hip_atomic_store(&ws->ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (lane < kMaxSlots) {
         __hip_atomic_store(&ws->slot[lane].bits, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(&ws->slot[lane].ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+}
+
+// `io2` / `pre2`: a second tensor role fed by the same amax (one source tensor quantised to both formats).
+__device__ inline void finalize_wave(Workspace* ws, const ScalarIO& io, int mode, const EpiloguePrefetch& pre,
+                                     const ScalarIO* io2 = nullptr, const EpiloguePrefetch* pre2 = nullptr) {
+    const uint32_t bits = collect_amax(ws);
+    bookkeep(bits, io, mode, pre);
+    if (io2) bookkeep(bits, *io2, mode, *pre2);
+    clear_workspace(ws);
 }
 
 // `bid` of `nblocks`: this workgroup's place among the workgroups that reduce the same tensor (the whole grid,
@@ -213,7 +241,8 @@ __device__ inline void finalize_wave(Workspace* ws, const ScalarIO& io, int mode
 template <int THREADS>
 __device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, const ScalarIO& io, int mode,
                                             const EpiloguePrefetch& pre, uint32_t bid = blockIdx.x,
-                                            uint32_t nblocks = gridDim.x) {
+                                            uint32_t nblocks = gridDim.x, const ScalarIO* io2 = nullptr,
+                                            const EpiloguePrefetch* pre2 = nullptr) {
     __shared__ uint32_t s_part[THREADS / 64];
     __shared__ bool s_last;
     const uint32_t wm = wave_max_u32(m_f32bits);
@@ -242,7 +271,7 @@ __device__ inline void publish_and_finalize(uint32_t m_f32bits, Workspace* ws, c
     __syncthreads();
     // the epilogue runs on the first wave of the block that drew the last ticket
     if (!s_last || threadIdx.x >= 64) return;
-    finalize_wave(ws, io, mode, pre);
+    finalize_wave(ws, io, mode, pre, io2, pre2);
 }
 
 // The same bookkeeping for maxima that another kernel (the fp8-output GEMM epilogue) left in the slots.
@@ -319,6 +348,54 @@ __global__ __launch_bounds__(kFlatThreads) void quant_flat_kernel(const typename
                                                               const float* __restrict__ scale_ptr, Workspace* ws,
                                                               ScalarIO io) {
     quant_flat_body<S, F, MODE>(x, n_vec, n, out, scale_ptr, ws, io, blockIdx.x, gridDim.x);
+}
+
+// One source tensor, both formats, one pass: the fused delayed-scaling step of an e4m3 role and an e5m2 role that
+// quantise the same tensor (4 bytes per bf16 element instead of 2 x 3).  The amax is shared; each role has its own
+// scale, history and output.
+template <typename S>
+__global__ __launch_bounds__(kFlatThreads) void quant_flat_dual_kernel(const typename ElemOf<S>::type* __restrict__ x,
+                                                                   int64_t n_vec, int64_t n, uint8_t* __restrict__ out0,
+                                                                   uint8_t* __restrict__ out1, Workspace* ws, ScalarIO io0,
+                                                                   ScalarIO io1) {
+    typedef Src<S> L;
+    const float s0 = *io0.scale_state, s1 = *io1.scale_state;
+    const bool d0 = degenerate_scale(s0), d1 = degenerate_scale(s1);
+    const EpiloguePrefetch pre0 = prefetch_epilogue(io0, kModeDelayed);
+    const EpiloguePrefetch pre1 = prefetch_epilogue(io1, kModeDelayed);
+    uint32_t m_run = 0;
+    const int64_t stride = (int64_t)gridDim.x * kFlatThreads;
+    int64_t i = (int64_t)blockIdx.x * kFlatThreads + threadIdx.x;
+    for (; i + stride < n_vec; i += 2 * stride) {
+        float v0[16], v1[16];
+        uint32_t m0, m1;
+        L::load16(x + i * kVec, v0, m0);
+        L::load16(x + (i + stride) * kVec, v1, m1);
+        m_run = m0 > m_run ? m0 : m_run;
+        m_run = m1 > m_run ? m1 : m_run;
+        const bool n0 = L::has_nan(m0), n1 = L::has_nan(m1);
+        __builtin_nontemporal_store(encode16<kE4M3>(v0, s0, d0 || n0), reinterpret_cast<u4*>(out0 + i * kVec));
+        __builtin_nontemporal_store(encode16<kE5M2>(v0, s1, d1 || n0), reinterpret_cast<u4*>(out1 + i * kVec));
+        __builtin_nontemporal_store(encode16<kE4M3>(v1, s0, d0 || n1), reinterpret_cast<u4*>(out0 + (i + stride) * kVec));
+        __builtin_nontemporal_store(encode16<kE5M2>(v1, s1, d1 || n1), reinterpret_cast<u4*>(out1 + (i + stride) * kVec));
+    }
+    if (i < n_vec) {
+        float v0[16];
+        uint32_t m0;
+        L::load16(x + i * kVec, v0, m0);
+        m_run = m0 > m_run ? m0 : m_run;
+        const bool n0 = L::has_nan(m0);
+        __builtin_nontemporal_store(encode16<kE4M3>(v0, s0, d0 || n0), reinterpret_cast<u4*>(out0 + i * kVec));
+        __builtin_nontemporal_store(encode16<kE5M2>(v0, s1, d1 || n0), reinterpret_cast<u4*>(out1 + i * kVec));
+    }
+    for (int64_t j = n_vec * kVec + (int64_t)blockIdx.x * kFlatThreads + threadIdx.x; j < n; j += stride) {
+        uint32_t m;
+        const float xv = L::load1(x + j, m);
+        m_run = m > m_run ? m : m_run;
+        out0[j] = encode1<kE4M3>(xv, s0);
+        out1[j] = encode1<kE5M2>(xv, s1);
+    }
+    publish_and_finalize<kFlatThreads>(L::to_f32_bits(m_run), ws, io0, kModeDelayed, pre0, blockIdx.x, gridDim.x, &io1, &pre1);
 }
 
 // Several tensors, one launch (the fused delayed-scaling step of each): the workgroups of tensor t follow those of
@@ -440,10 +517,12 @@ __device__ __forceinline__ float decode1(uint32_t b) {
     else return __builtin_amdgcn_cvt_f32_bf8((int)b, 0);
 }
 
+// `is_inverse`: scale_ptr holds 1 / scale already (the form tex.cast_from_fp8 is handed, src/nanotron/fp8/tensor.py:74)
 template <int F, int OUT>
 __global__ __launch_bounds__(kThreads) void dequant_kernel(const uint8_t* __restrict__ in, int64_t n,
-                                                           const float* __restrict__ scale_ptr, void* __restrict__ out) {
-    const float inv = 1.0f / *scale_ptr;
+                                                           const float* __restrict__ scale_ptr, void* __restrict__ out,
+                                                           int is_inverse) {
+    const float inv = is_inverse ? *scale_ptr : 1.0f / *scale_ptr;
     const int64_t stride = (int64_t)gridDim.x * kThreads;
     for (int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x; j < n; j += stride) {
         float v = decode1<F>(in[j]) * inv;
@@ -493,6 +572,10 @@ static int grid_for(int64_t work_items, int threads = kThreads, int per_cu_block
     return (int)(want < cap ? want : cap);
 }
 
+// The launch macro reports through the thread's last-error slot.  hipGetLastError() reads and clears it; an error
+// left there by an unrelated earlier call of this thread is dropped by clear_stale_error() before a launch, so that
+// check_launch() speaks for this library's launch only.
+static void clear_stale_error() { (void)hipGetLastError(); }
 static int check_launch() { return hipGetLastError() == hipSuccess ? NTFP8_OK : NTFP8_ERR_LAUNCH; }
 
 template <typename S, int F>
@@ -562,6 +645,7 @@ static bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_
 // mode: kModeAmaxOnly / kModeCastOnly / kModeDelayed.  out_t may be NULL.
 int run_quant(int mode, const void* x, int x_dtype, int64_t rows, int64_t cols, int fmt, uint8_t* out, uint8_t* out_t,
               const float* scale_ptr, Workspace* ws, const ScalarIO& io, hipStream_t st) {
+    clear_stale_error();
     const int64_t n = rows * cols;
     if (mode != kModeAmaxOnly && out_t != nullptr) {
         const bool tile_ok = rows % kTile == 0 && cols % kTile == 0 && aligned(x, 16) && aligned(out_t, 16) &&
@@ -583,6 +667,7 @@ int run_quant(int mode, const void* x, int x_dtype, int64_t rows, int64_t cols, 
 
 template <typename S, int F>
 static int launch_flat_multi(const QuantDesc* const* q, int count, hipStream_t st) {
+    clear_stale_error();
     MultiQuant Q = {};
     Q.count = count;
     int blocks = 0;
@@ -643,10 +728,36 @@ int run_quant_delayed_batch(const QuantDesc* q, int count, hipStream_t st) {
     return NTFP8_OK;
 }
 
-int run_dequant(const void* in, int fmt, const float* scale, int64_t n, void* out, int out_dtype, hipStream_t st) {
+// Both formats from one pass over x (flat layout only).
+int run_quant_dual(const void* x, int x_dtype, int64_t n, uint8_t* out_e4m3, uint8_t* out_e5m2, Workspace* ws,
+                   const ScalarIO& io_e4m3, const ScalarIO& io_e5m2, hipStream_t st) {
+    clear_stale_error();
+    const bool vec_ok = aligned(x, 16) && aligned(out_e4m3, 16) && aligned(out_e5m2, 16);
+    const int64_t n_vec = vec_ok ? n / kVec : 0;
+    const int grid = grid_for(n_vec > 0 ? (n_vec + 1) / 2 : n, kFlatThreads, 1);
+    switch (x_dtype) {
+        case NTFP8_F32:
+            hipLaunchKernelGGL((quant_flat_dual_kernel<float>), dim3(grid), dim3(kFlatThreads), 0, st,
+                               static_cast<const float*>(x), n_vec, n, out_e4m3, out_e5m2, ws, io_e4m3, io_e5m2);
+            break;
+        case NTFP8_F16:
+            hipLaunchKernelGGL((quant_flat_dual_kernel<f16_tag>), dim3(grid), dim3(kFlatThreads), 0, st,
+                               static_cast<const uint16_t*>(x), n_vec, n, out_e4m3, out_e5m2, ws, io_e4m3, io_e5m2);
+            break;
+        default:
+            hipLaunchKernelGGL((quant_flat_dual_kernel<bf16_tag>), dim3(grid), dim3(kFlatThreads), 0, st,
+                               static_cast<const uint16_t*>(x), n_vec, n, out_e4m3, out_e5m2, ws, io_e4m3, io_e5m2);
+            break;
+    }
+    return check_launch();
+}
+
+int run_dequant(const void* in, int fmt, const float* scale, int is_inverse, int64_t n, void* out, int out_dtype,
+                hipStream_t st) {
+    clear_stale_error();
     const int grid = grid_for(n);
     const uint8_t* p = static_cast<const uint8_t*>(in);
-#define NT_DQ(F, O) hipLaunchKernelGGL((dequant_kernel<F, O>), dim3(grid), dim3(kThreads), 0, st, p, n, scale, out)
+#define NT_DQ(F, O) hipLaunchKernelGGL((dequant_kernel<F, O>), dim3(grid), dim3(kThreads), 0, st, p, n, scale, out, is_inverse)
     if (fmt == kE4M3) {
         if (out_dtype == NTFP8_F32) NT_DQ(kE4M3, NTFP8_F32);
         else if (out_dtype == NTFP8_F16) NT_DQ(kE4M3, NTFP8_F16);
@@ -661,6 +772,7 @@ int run_dequant(const void* in, int fmt, const float* scale, int64_t n, void* ou
 }
 
 int run_transpose(const void* in, int64_t rows, int64_t cols, void* out, hipStream_t st) {
+    clear_stale_error();
     const int64_t tiles = ((rows + 63) / 64) * ((cols + 63) / 64);
     if (tiles > 0x7fffffff) return NTFP8_ERR_SIZE;
     hipLaunchKernelGGL(transpose_kernel, dim3((int)tiles), dim3(kThreads), 0, st, static_cast<const uint8_t*>(in), rows,
@@ -669,12 +781,14 @@ int run_transpose(const void* in, int64_t rows, int64_t cols, void* out, hipStre
 }
 
 int run_amax_finalize(Workspace* ws, const ScalarIO& io, hipStream_t st) {
+    clear_stale_error();
     hipLaunchKernelGGL(amax_finalize_kernel, dim3(1), dim3(64), 0, st, ws, io);
     return check_launch();
 }
 
 int run_update_scale(const float* amax, const float* old_scale, int fmt, int margin, float* out, int64_t n,
                      hipStream_t st) {
+    clear_stale_error();
     const int64_t blocks = (n + 255) / 256;
     if (blocks > 0x7fffffff) return NTFP8_ERR_SIZE;
     hipLaunchKernelGGL(update_scale_kernel, dim3((int)blocks), dim3(256), 0, st, amax, old_scale, fmt, margin, out, n);

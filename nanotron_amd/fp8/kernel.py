@@ -10,17 +10,33 @@ _FMT = {DTypes.FP8E4M3: nt.E4M3, DTypes.FP8E5M2: nt.E5M2}
 _OUT_FMT = {DTypes.FP8E4M3: nt.OUT_E4M3, DTypes.FP8E5M2: nt.OUT_E5M2}
 
 
-def _gemm_nt(a: FP8Tensor, b: FP8Tensor, out_dtype: torch.dtype, accumulate_into: Optional[torch.Tensor]):
-    """D[M,N] = A[M,K] . B[N,K]^T, descaled (te_gemm's TN form, src/nanotron/fp8/kernel.py:46-68)."""
+def _bytes_and_meta(t: FP8Tensor):
+    """(contiguous uint8 tensor, meta) of an fp8 operand.  The meta is a Python attribute of the FP8Tensor object: a
+    copy made by `.contiguous()` (of a view such as a slice or `.t()`) does not carry it, so it is read first."""
+    meta = t.fp8_meta
+    raw = t.as_subclass(torch.Tensor)
+    return (raw if raw.is_contiguous() else raw.contiguous()), meta
+
+
+def _check_bias(bias: torch.Tensor, N: int, dev) -> torch.Tensor:
+    assert bias.dim() == 1 and bias.shape[0] == N and bias.device == dev, (tuple(bias.shape), N)
+    assert bias.dtype in nt.TORCH_TO_NT, f"unsupported bias dtype {bias.dtype}"
+    return bias.detach().contiguous()
+
+
+def _gemm_nt(a: FP8Tensor, b: FP8Tensor, out_dtype: torch.dtype, accumulate_into: Optional[torch.Tensor],
+             bias: Optional[torch.Tensor] = None):
+    """D[M,N] = A[M,K] . B[N,K]^T, descaled (te_gemm's TN form, src/nanotron/fp8/kernel.py:46-68); with `bias`
+    [N] added to the descaled fp32 result before the single rounding (te_gemm's bias argument, which the
+    reference leaves empty, kernel.py:29-32)."""
+    if bias is not None:
+        return _gemm_nt_batch([(a, b, out_dtype, accumulate_into, False, bias)])[0]
     assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[1], (tuple(a.shape), tuple(b.shape))
     M, K = a.shape
     N = b.shape[0]
     dev = a.device
-    if not a.is_contiguous():
-        a = a.contiguous()
-    if not b.is_contiguous():
-        b = b.contiguous()
-    ma, mb = a.fp8_meta, b.fp8_meta
+    a, ma = _bytes_and_meta(a)
+    b, mb = _bytes_and_meta(b)
     if accumulate_into is not None:
         assert accumulate_into.dtype == torch.float32 and accumulate_into.shape == (M, N)
         assert accumulate_into.is_contiguous() and accumulate_into.device == dev
@@ -35,7 +51,7 @@ def _gemm_nt(a: FP8Tensor, b: FP8Tensor, out_dtype: torch.dtype, accumulate_into
 
 
 def _gemm_nt_fp8(a: FP8Tensor, b: FP8Tensor, dtype: DTypes, state: Optional[DelayedScaling],
-                 with_transpose: bool) -> FP8Tensor:
+                 with_transpose: bool, bias: Optional[torch.Tensor] = None) -> FP8Tensor:
     """FP8Tensor(_gemm_nt(a, b, float32), dtype, state=state, with_transpose=with_transpose), bit for bit, with the
     fp32 result never written to memory: the GEMM epilogue casts with the scale `state` holds from earlier steps,
     leaves max|result| behind, and a one-wave kernel turns that into amax, history roll and next scale.
@@ -46,18 +62,17 @@ def _gemm_nt_fp8(a: FP8Tensor, b: FP8Tensor, dtype: DTypes, state: Optional[Dela
 
     assert dtype in _OUT_FMT, f"{dtype} is not an FP8 format"
     if state is None or not state.initialised:
-        return FP8Tensor(_gemm_nt(a, b, torch.float32, None), dtype, state=state, with_transpose=with_transpose)
+        return FP8Tensor(_gemm_nt(a, b, torch.float32, None, bias), dtype, state=state, with_transpose=with_transpose)
     assert state.dtype == dtype, "delayed-scaling state was created for another format"
     assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[1], (tuple(a.shape), tuple(b.shape))
     M, K = a.shape
     N = b.shape[0]
     dev = a.device
     assert state._buf.device == dev
-    if not a.is_contiguous():
-        a = a.contiguous()
-    if not b.is_contiguous():
-        b = b.contiguous()
-    ma, mb = a.fp8_meta, b.fp8_meta
+    a, ma = _bytes_and_meta(a)
+    b, mb = _bytes_and_meta(b)
+    if bias is not None:
+        bias = _check_bias(bias, N, dev)
     out = torch.empty((M, N), dtype=torch.uint8, device=dev)
     out_t = torch.empty((N, M), dtype=torch.uint8, device=dev) if with_transpose else None
     scalars = torch.empty(2, dtype=torch.float32, device=dev)  # [amax, scale used]
@@ -69,6 +84,8 @@ def _gemm_nt_fp8(a: FP8Tensor, b: FP8Tensor, dtype: DTypes, state: Optional[Dela
     d[0].M, d[0].N, d[0].K = M, N, K
     d[0].fmt_a, d[0].fmt_b, d[0].d_dtype, d[0].accumulate = _FMT[ma.dtype], _FMT[mb.dtype], _OUT_FMT[dtype], 0
     d[0].scale_d, d[0].D_t, d[0].amax_workspace = state_p, nt.ptr(out_t), ws.data_ptr()
+    if bias is not None:
+        d[0].bias, d[0].bias_dtype = bias.data_ptr(), nt.TORCH_TO_NT[bias.dtype]
     nt.check(nt.lib.ntfp8_gemm_batch(d, 1, st), "ntfp8_gemm_batch")
     nt.check(nt.lib.ntfp8_amax_finalize(ws.data_ptr(), _FMT[dtype], state.margin, state_p, state_p + 4, state.history_len,
                                         scalars.data_ptr(), scalars.data_ptr() + 4, st), "ntfp8_amax_finalize")
@@ -102,42 +119,43 @@ def needs_transposed_copy(rows: int, cols: int, other: int = 4096) -> bool:
 
 
 def _gemm_nt_batch(problems):
-    """Several independent `_gemm_nt` problems, given as tuples (a, b, out_dtype, accumulate_into[, b_transposed]),
-    in one call of the library: GEMMs with the same operand formats share launches.  With `b_transposed` the
-    tensor `b` is the [K, N] transpose of the operand.  Returns the outputs in order."""
+    """Several independent `_gemm_nt` problems, given as tuples (a, b, out_dtype, accumulate_into[, b_transposed[,
+    bias]]), in one call of the library: GEMMs with the same operand formats share launches.  With `b_transposed`
+    the tensor `b` is the [K, N] transpose of the operand.  Returns the outputs in order."""
     descs = (nt.GemmDesc * len(problems))()
     outs, keep = [], []
     dev = problems[0][0].device
     for d, prob in zip(descs, problems):
         a, b, out_dtype, accumulate_into = prob[:4]
         bt = bool(prob[4]) if len(prob) > 4 else False
+        bias = prob[5] if len(prob) > 5 else None
         assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0 if bt else 1], (tuple(a.shape), tuple(b.shape), bt)
         assert a.device == dev and b.device == dev
         M, K = a.shape
         N = b.shape[1 if bt else 0]
-        if not a.is_contiguous():
-            a = a.contiguous()
-        if not b.is_contiguous():
-            b = b.contiguous()
-        ma, mb = a.fp8_meta, b.fp8_meta
+        a, ma = _bytes_and_meta(a)
+        b, mb = _bytes_and_meta(b)
         if accumulate_into is not None:
             assert accumulate_into.dtype == torch.float32 and accumulate_into.shape == (M, N)
             assert accumulate_into.is_contiguous() and accumulate_into.device == dev
             out, acc = accumulate_into, 1
         else:
             out, acc = torch.empty((M, N), dtype=out_dtype, device=dev), 0
+        if bias is not None:
+            bias = _check_bias(bias, N, dev)
+            d.bias, d.bias_dtype = bias.data_ptr(), nt.TORCH_TO_NT[bias.dtype]
         d.A, d.scale_a, d.B, d.scale_b, d.D = a.data_ptr(), ma.scale.data_ptr(), b.data_ptr(), mb.scale.data_ptr(), out.data_ptr()
         d.M, d.N, d.K = M, N, K
         d.fmt_a, d.fmt_b, d.d_dtype, d.accumulate = _FMT[ma.dtype], _FMT[mb.dtype], nt.TORCH_TO_NT[out.dtype], acc
         d.b_transposed = 1 if bt else 0
         outs.append(out)
-        keep.append((a, b))
+        keep.append((a, b, bias))
     nt.check(nt.lib.ntfp8_gemm_batch(descs, len(problems), nt.stream_ptr(dev)), "ntfp8_gemm_batch")
     return outs
 
 
 def _operands(mat_a: FP8Tensor, transpose_a: bool, mat_b: FP8Tensor, transpose_b: bool,
-              accumulate_into: Optional[torch.Tensor] = None):
+              accumulate_into: Optional[torch.Tensor] = None, allow_bt: bool = True):
     """(A, B, b_transposed) of the library's D = A . B^T for the reference's D = op_b(B) . op_a(A) (kernel.py:43-44).
 
     Where the reference transposes mat_a (tex.fp8_transpose, kernel.py:43) the library can read it as it is
@@ -150,7 +168,7 @@ def _operands(mat_a: FP8Tensor, transpose_a: bool, mat_b: FP8Tensor, transpose_b
     if transpose_a:
         return b_, mat_a, False
     aligned = all(t is None or t.data_ptr() % 16 == 0 for t in (mat_a, b_, accumulate_into))   # 16-byte loads / stores
-    if getattr(mat_a, "_transposed", None) is None and mat_a.dim() == 2 and mat_a.is_contiguous() and aligned and \
+    if allow_bt and getattr(mat_a, "_transposed", None) is None and mat_a.dim() == 2 and mat_a.is_contiguous() and aligned and \
             b_transposed_supported(b_.shape[0], mat_a.shape[1], mat_a.shape[0]):
         return b_, mat_a, True
     return b_, mat_a.transposed(), False
@@ -181,6 +199,7 @@ def fp8_matmul_kernel(
     accumulate_into: Optional[torch.Tensor] = None,
     out_state: Optional[DelayedScaling] = None,
     out_with_transpose: bool = False,
+    bias: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """D = op_b(B) . op_a(A) * (1/scale_a)(1/scale_b), op_x(X) = X^T if transpose_x else X
     (reference: src/nanotron/fp8/kernel.py:9-70; the operator meaning follows from its fixed
@@ -193,7 +212,10 @@ def fp8_matmul_kernel(
     `accumulate_into` (fp32, contiguous) receives D added in place before any rounding.
     `out_dtype=DTypes.FP8E4M3 / FP8E5M2` returns D as an FP8Tensor ("return an fp8 tensor as output", the TODO at
     src/nanotron/fp8/linear.py:63-64), quantised with the delayed-scaling state `out_state` in the GEMM's epilogue
-    and, with `out_with_transpose`, carrying its transposed copy."""
+    and, with `out_with_transpose`, carrying its transposed copy.
+    `bias` (one value per column of D, fp32 / fp16 / bf16) is added to the descaled fp32 result before the single
+    rounding to the output type: the bias argument of te_gemm that the reference leaves empty (kernel.py:29-32).
+    For an fp32 output this equals `D + bias` bit for bit."""
     assert mat_a.device != torch.device("cpu") and mat_b.device != torch.device("cpu"), \
         "The tensors must be on a CUDA device in order to use the FP8 kernel!!"
     assert hasattr(mat_a, "fp8_meta") and hasattr(mat_b, "fp8_meta"), "operands must be FP8Tensors"
@@ -201,8 +223,8 @@ def fp8_matmul_kernel(
         assert accumulate_into is None, "an fp8 output cannot accumulate"
         a_ = mat_a if transpose_a else mat_a.transposed()  # kernel.py:43
         b_ = mat_b.transposed() if transpose_b else mat_b  # kernel.py:44
-        return _gemm_nt_fp8(b_, a_, out_dtype, out_state, out_with_transpose)
-    A, B, bt = _operands(mat_a, transpose_a, mat_b, transpose_b, accumulate_into)
+        return _gemm_nt_fp8(b_, a_, out_dtype, out_state, out_with_transpose, bias)
+    A, B, bt = _operands(mat_a, transpose_a, mat_b, transpose_b, accumulate_into, allow_bt=bias is None)
     if bt:
         return _gemm_nt_batch([(A, B, out_dtype or torch.float32, accumulate_into, True)])[0]
-    return _gemm_nt(A, B, out_dtype or torch.float32, accumulate_into)
+    return _gemm_nt(A, B, out_dtype or torch.float32, accumulate_into, bias)

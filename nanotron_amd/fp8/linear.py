@@ -26,12 +26,15 @@ class FP8Linear(nn.Linear):
     Positional signature as the reference.  Keyword-only extensions, all defaulting to the
     reference's behaviour: `dtype` (of the master weight and bias, as nn.Linear's), `out_dtype`
     (None = fp32 output, kernel.py:24,28; `DTypes.FP8E4M3` / `FP8E5M2` = the output is returned as an
-    FP8Tensor, the TODO at linear.py:63-64: forward only, no bias, quantised in the GEMM epilogue with the
-    delayed-scaling role "output", its transposed copy included if `fp8_output_transpose`), `delayed_scaling`
+    FP8Tensor, the TODO at linear.py:63-64, quantised in the GEMM epilogue with the delayed-scaling role "output",
+    its transposed copy included if `fp8_output_transpose`; it carries a gradient handle, so that a following
+    FP8Linear back-propagates into this one, see _FP8Matmul), `delayed_scaling`
     (False = scale every tensor from its own amax), `amax_history_len`, `margin`,
     `accumulate_grad` (False = `weight.grad` is overwritten each backward, linear.py:110; True =
     the wgrad GEMM adds into the existing fp32 gradient in its epilogue).  With a bf16 / fp16
-    master weight the fp32 weight gradient is stored as `weight.main_grad` instead of `.grad`."""
+    master weight the fp32 weight gradient is stored as `weight.main_grad` instead of `.grad`.
+    The bias is added inside the GEMM epilogue (the TODO at linear.py:62).  In evaluation mode (`module.eval()`)
+    tensors are quantised with the scales the delayed-scaling roles hold and the roles are left untouched."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, device: Optional[torch.device] = None,
                  *, dtype: Optional[torch.dtype] = None, out_dtype: Union[torch.dtype, DTypes, None] = None,
@@ -41,8 +44,6 @@ class FP8Linear(nn.Linear):
         if isinstance(out_dtype, DTypes):
             if out_dtype not in (DTypes.FP8E4M3, DTypes.FP8E5M2):
                 raise ValueError(f"{out_dtype} is not an FP8 format")
-            if bias:
-                raise ValueError("an fp8 output is quantised inside the GEMM, before a bias could be added: use bias=False")
         self.out_dtype = out_dtype
         self.fp8_output_transpose = fp8_output_transpose
         self.accumulate_grad = accumulate_grad
@@ -170,44 +171,73 @@ class FP8Linear(nn.Linear):
         # phony tensor that makes autograd call our backward although the weight's gradient is
         # produced by the fp8 kernels, not by autograd (linear.py:56-60)
         phony = torch.empty(0, device=input.device, requires_grad=True)
-        output, _ = _FP8Matmul.apply(input, self.weight, self, phony)
-        output = output if self.bias is None else output + self.bias
+        # The bias goes into the GEMM's epilogue (the TODO at linear.py:62; for the fp32 output of the reference the
+        # result equals `output + self.bias`, linear.py:65, bit for bit) and an fp8 input produced by another
+        # FP8Linear brings the handle its gradient travels through (below).
+        output, aux = _FP8Matmul.apply(input, self.weight, self.fp8_meta, phony, self, self.bias,
+                                       getattr(input, "_grad_handle", None))
+        if isinstance(self.out_dtype, DTypes):
+            output._grad_handle = aux
         return output
 
 
 class _FP8Matmul(torch.autograd.Function):
     """Y = X.W^T forward; dX = dY.W and dW = dY^T.X backward, all three on the fp8 matrix cores
     (reference: src/nanotron/fp8/linear.py:69-112).  The backward computes the gradients its
-    docstring states (linear.py:92-96) for any shape and uses the real upstream gradient."""
+    docstring states (linear.py:92-96) for any shape and uses the real upstream gradient.
+
+    `apply(input, weight, fp8_meta, phony)` is the reference's call (linear.py:60): current scaling, fp32 output.
+    Three more positional arguments carry this build's extensions: `module` (the FP8Linear: output type, delayed
+    scaling roles, gradient accumulation), `bias` (added in the GEMM epilogue; its gradient is returned like any
+    other) and `input_handle`.
+
+    fp8 activations and autograd.  With `module.out_dtype` an FP8 format the output is an FP8Tensor, a uint8 tensor
+    that cannot carry a gradient.  The second output then is its *gradient handle*: a [tokens, out_features] tensor
+    of the high-precision type without memory of its own (one element, expanded), part of the autograd graph.  The
+    FP8Linear that consumes the FP8Tensor passes the handle along as `input_handle`; its backward returns dX as the
+    handle's gradient, and autograd delivers it to the producer's backward as the gradient of the output it stands
+    for.  So a chain FP8Linear(out_dtype=E4M3) -> FP8Linear trains without the activation ever leaving fp8."""
 
     @staticmethod
     @torch.no_grad()
-    def forward(ctx, input, weight, module: "FP8Linear", phony: torch.Tensor):
-        scaling = module.scaling
+    def forward(ctx, input, weight, fp8_meta, phony: torch.Tensor, module: Optional["FP8Linear"] = None,
+                bias: Optional[torch.Tensor] = None, input_handle: Optional[torch.Tensor] = None):
+        scaling = module.scaling if module is not None else None
+        update = module.training if module is not None else True   # evaluation passes leave the scaling state alone
         needs_wgrad = weight.requires_grad
-        ctx.in_dtype = input.dtype if type(input) == torch.Tensor else None
+        ctx.in_dtype = input.dtype if type(input) == torch.Tensor else (input_handle.dtype if input_handle is not None else None)
         ctx.in_shape = input.shape
+        ctx.has_handle = input_handle is not None
         if type(input) == torch.Tensor:
             x2d = input.reshape(-1, input.shape[-1])
             input = FP8Tensor(x2d, dtype=DTypes.FP8E4M3, state=scaling["input"] if scaling else None,
-                              with_transpose=needs_wgrad and needs_transposed_copy(x2d.shape[0], x2d.shape[1], weight.shape[0]))
-        ctx.save_for_backward(input, weight)
+                              with_transpose=needs_wgrad and needs_transposed_copy(x2d.shape[0], x2d.shape[1], weight.shape[0]),
+                              update_state=update)
+        ctx.save_for_backward(input, weight, bias)
         ctx.module = module
-        out_dtype = module.out_dtype or torch.float32
+        ctx.fp8_meta = fp8_meta
+        out_dtype = (module.out_dtype if module is not None else None) or torch.float32
+        gemm_bias = bias.detach() if bias is not None else None
 
         # FP8Tensor of the weight, not the FP8Parameter (linear.py:81-84)
         if isinstance(out_dtype, DTypes):
             # [tokens, out_features] whatever the input's leading dimensions: what the next layer's GEMM consumes
+            state = scaling["output"] if scaling else None
+            if state is not None and not update and state.initialised:
+                state = _frozen_copy(state)
             output = fp8_matmul_kernel(
                 mat_a=weight.data, transpose_a=True, mat_b=input, transpose_b=False, use_split_accumulator=False,
-                out_dtype=out_dtype, out_state=scaling["output"] if scaling else None,
-                out_with_transpose=module.fp8_output_transpose,
+                out_dtype=out_dtype, out_state=state, out_with_transpose=module.fp8_output_transpose, bias=gemm_bias,
             )
             ctx.mark_non_differentiable(output)
-            return output, phony
+            hp = weight.dtype if weight.dtype in (torch.float32, torch.float16, torch.bfloat16) else torch.float32
+            handle = torch.zeros(1, dtype=hp, device=output.device).expand(output.shape)
+            ctx.fp8_out = True
+            return output, handle
+        ctx.fp8_out = False
         output = fp8_matmul_kernel(
             mat_a=weight.data, transpose_a=True, mat_b=input, transpose_b=False, use_split_accumulator=False,
-            out_dtype=out_dtype,
+            out_dtype=out_dtype, bias=gemm_bias,
         )
         if len(ctx.in_shape) != 2:
             output = output.reshape(*ctx.in_shape[:-1], output.shape[-1])
@@ -215,16 +245,32 @@ class _FP8Matmul(torch.autograd.Function):
 
     @staticmethod
     @torch.no_grad()
-    def backward(ctx, grad_output: torch.Tensor, grad_phony: torch.Tensor) -> Tuple[torch.Tensor, None, None, None]:
-        input, weight = ctx.saved_tensors
+    def backward(ctx, grad_output: torch.Tensor, grad_aux: torch.Tensor):
+        input, weight, bias = ctx.saved_tensors
         module = ctx.module
-        scaling = module.scaling
+        scaling = module.scaling if module is not None else None
+        none = (None,) * 7
+        if ctx.fp8_out:
+            grad_output = grad_aux   # the gradient of the fp8 output arrives through its handle
+        if grad_output is None:
+            return none
+
+        grad_bias = None
+        if bias is not None and ctx.needs_input_grad[5]:
+            # what autograd does for `output + bias` (linear.py:65): the gradient summed over the tokens (in fp32)
+            g_hp = grad_output
+            if type(g_hp) != torch.Tensor:
+                from nanotron_amd.fp8.tensor import convert_tensor_from_fp8
+
+                g_hp = convert_tensor_from_fp8(g_hp, g_hp.fp8_meta, bias.dtype)
+            grad_bias = g_hp.reshape(-1, g_hp.shape[-1]).sum(0, dtype=torch.float32).to(bias.dtype)
 
         if type(grad_output) == torch.Tensor:
             g2d = grad_output.reshape(-1, grad_output.shape[-1]).contiguous()
             grad_output = FP8Tensor(g2d, dtype=DTypes.FP8E5M2, state=scaling["output_grad"] if scaling else None,
                                     with_transpose=weight.requires_grad)
 
+        wants_dx = ctx.needs_input_grad[0] or (ctx.has_handle and ctx.needs_input_grad[6])
         grad_input = None
         # dX[M,K] = dY[M,N] . W[N,K]
         dgrad = dict(mat_a=weight.data, transpose_a=False, mat_b=grad_output, transpose_b=False, use_split_accumulator=True,
@@ -236,19 +282,19 @@ class _FP8Matmul(torch.autograd.Function):
             # beside the parameter as `.main_grad`, the fp32 master-gradient buffer an optimizer reads.
             slot = "grad" if weight.dtype == torch.float32 else "main_grad"
             acc = None
-            if module.accumulate_grad:
+            if module is not None and module.accumulate_grad:
                 prev = getattr(weight, slot, None)
                 if prev is not None and prev.dtype == torch.float32:
                     acc = prev
             wgrad = dict(mat_a=input, transpose_a=False, mat_b=grad_output, transpose_b=True, use_split_accumulator=True,
                          accumulate_into=acc)
         grad_weight = None
-        if ctx.needs_input_grad[0] and wgrad is not None:
+        if wants_dx and wgrad is not None:
             # the two GEMMs are independent: issued together they share kernel launches
             grad_input, grad_weight = fp8_matmul_pair(
                 {k: v for k, v in dgrad.items() if k != "use_split_accumulator"},
                 {k: v for k, v in wgrad.items() if k != "use_split_accumulator"})
-        elif ctx.needs_input_grad[0]:
+        elif wants_dx:
             grad_input = fp8_matmul_kernel(**dgrad)
         elif wgrad is not None:
             grad_weight = fp8_matmul_kernel(**wgrad)
@@ -257,4 +303,15 @@ class _FP8Matmul(torch.autograd.Function):
         if grad_weight is not None:
             setattr(weight, slot, grad_weight)
 
-        return grad_input, None, None, None
+        if ctx.has_handle:   # the input was an fp8 activation: its gradient goes to the handle that stands for it
+            return None, None, None, None, None, grad_bias, grad_input
+        return grad_input, None, None, None, None, grad_bias, None
+
+
+def _frozen_copy(state: DelayedScaling) -> DelayedScaling:
+    """A throw-away copy of a delayed-scaling state: the fp8-output GEMM of an evaluation pass casts with the held
+    scale and does its bookkeeping on the copy."""
+    c = DelayedScaling(state.dtype, state.history_len, state.margin, state._buf.device)
+    c._buf.copy_(state._buf)
+    c.initialised = state.initialised
+    return c

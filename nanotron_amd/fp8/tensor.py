@@ -71,14 +71,19 @@ class FP8Tensor(torch.Tensor):
 
     `FP8Tensor(tensor, dtype)` is the reference call (current scaling).  Keyword-only extensions:
     `state` selects delayed scaling for a tensor role, `with_transpose` also produces the
-    transposed bytes in the same pass (what the backward GEMMs consume)."""
+    transposed bytes in the same pass (what the backward GEMMs consume), `update_state=False` quantises with the
+    scale `state` holds but leaves the state as it is (evaluation passes between training steps)."""
 
     def __new__(cls, tensor: torch.Tensor, dtype: DTypes, *, state: Optional[DelayedScaling] = None,
-                with_transpose: bool = False, margin: int = 0) -> "FP8Tensor":
+                with_transpose: bool = False, margin: int = 0, update_state: bool = True) -> "FP8Tensor":
         assert isinstance(tensor, torch.Tensor), "tensor must be a tensor"
         assert tensor.dtype not in FP8_DTYPES, "The tensor already quantized to FP8"
         assert tensor.device != torch.device("cpu"), "FP8Tensor only supports CUDA device"
         assert isinstance(dtype, DTypes)
+        if state is not None and not update_state:
+            if state.initialised:
+                return cast_with_scale(tensor, state.scale, dtype, with_transpose=with_transpose)
+            return _quantize(cls, tensor, dtype, None, with_transpose, state.margin)
         return _quantize(cls, tensor, dtype, state, with_transpose, margin)
 
     def transposed(self) -> "FP8Tensor":

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(nt.lib, n), f"{n} declared in include/ntfp8.h but not exported"
         assert n in nt.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(nt.SIGNATURES) == names
-    assert nt.version() == 1
+    assert nt.version() == 2
     assert nt.strerror(0) == "ok" and "NULL" in nt.strerror(-1)
 
 
@@ -173,7 +173,53 @@ def test_fp8_output_and_transposed_operand_requests_are_validated_before_any_lau
     assert L.ntfp8_amax_finalize(P, 0, 0, P + 4096, None, 4, P + 256, None, None) == -3           # length without a history
     assert L.ntfp8_amax_finalize(P, 0, 500, P + 4096, None, 0, P + 256, None, None) == -3
     assert L.ntfp8_amax_finalize(P, 0, 0, P + 4098, None, 0, P + 256, None, None) == -4
-    assert ctypes.sizeof(nt.GemmDesc) == 112
+    assert ctypes.sizeof(nt.GemmDesc) == 128
+    # bias: dtype, alignment, overlap with the output, not together with a transposed B operand
+    B0 = P + (5 << 20)
+    assert L.ntfp8_gemm_batch(desc(bias=B0, bias_dtype=7), 1, None) == -2
+    assert L.ntfp8_gemm_batch(desc(bias=B0 + 2, bias_dtype=0), 1, None) == -4
+    assert L.ntfp8_gemm_batch(desc(bias=P + (3 << 20) + 128, bias_dtype=2), 1, None) == -7
+    assert L.ntfp8_gemm_batch(desc(bias=B0, bias_dtype=2, b_transposed=1), 1, None) == -5
+
+
+def test_a_failed_batch_has_launched_nothing():
+    """A problem no kernel serves is found before the first launch: the call fails as a whole, so a binder that
+    falls back (transposed copy + ntfp8_gemm) never adds an accumulated gradient twice.  Proven on the host: the
+    first problem's pointers are fake, so a launch of it would fault; the call must return the code instead."""
+    from nanotron_amd import _native as nt
+
+    P = 0x100000
+    d = (nt.GemmDesc * 2)()
+    for i, (m, n, k, bt) in enumerate([(512, 512, 512, 0), (256, 250, 256, 1)]):   # fine; transposed B with N % 16 != 0
+        base = P + i * (16 << 20)
+        d[i].A, d[i].scale_a, d[i].B, d[i].scale_b, d[i].D = base, base + (1 << 20), base + (2 << 20), base + (1 << 20) + 64, base + (3 << 20)
+        d[i].M, d[i].N, d[i].K, d[i].fmt_a, d[i].fmt_b, d[i].d_dtype, d[i].accumulate = m, n, k, 0, 0, 0, 1 - i
+        d[i].b_transposed = bt
+    assert nt.lib.ntfp8_gemm_batch(d, 2, None) == -5
+
+
+def test_new_entry_points_validate_on_the_host():
+    from nanotron_amd import _native as nt
+
+    L = nt.lib
+    P = 0x300000
+    # tex-shaped cast: amax / scale_inv bookkeeping needs the workspace
+    assert L.ntfp8_te_cast_to_fp8(None, 2, 16, P, None, None, 0, P + 4096, None, None) == -1
+    assert L.ntfp8_te_cast_to_fp8(P, 2, 16, P + 8192, P + 8256, None, 0, P + 4096, None, None) == -1
+    assert L.ntfp8_te_cast_to_fp8(P, 2, 0, P + 8192, None, None, 0, P + 4096, None, None) == -3
+    assert L.ntfp8_te_cast_to_fp8(P, 2, 16, P + 8192, P + 8258, None, 0, P + 4096, P + 16384, None) == -4
+    assert L.ntfp8_te_cast_to_fp8(P, 2, 16, P + 8192, None, None, 3, P + 4096, None, None) == -2
+    assert L.ntfp8_te_cast_to_fp8(P, 2, 16, P + 8192, None, None, 0, P + 8, None, None) == -7
+    assert L.ntfp8_cast_from_fp8_scale_inv(P, 0, None, 16, P + 4096, 0, None) == -1
+    assert L.ntfp8_cast_from_fp8_scale_inv(P, 0, P + 8192, 16, P + 4096, 9, None) == -2
+    # both formats in one pass
+    args = dict(x=P, x_dtype=2, n=64, margin=0, s0=P + 4096, h0=P + 4100, s1=P + 4200, h1=P + 4204, hl=16, amax=P + 4400,
+                u0=None, u1=None, o0=P + 8192, o1=P + 12288, ws=P + 16384)
+    call = lambda **kw: L.ntfp8_quantize_delayed_dual(*[{**args, **kw}[k] for k in args], None)
+    assert call(o1=None) == -1 and call(ws=None) == -1
+    assert call(n=0) == -3 and call(hl=0) == -3
+    assert call(s1=P + 4202) == -4
+    assert call(s1=P + 4096) == -7 and call(o1=P + 8192 + 16) == -7 and call(o0=P + 8) == -7
 
 
 def test_host_policy_for_transposed_copies():

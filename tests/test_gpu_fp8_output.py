@@ -218,8 +218,10 @@ def test_two_linears_chained_through_an_fp8_activation():
         hq = O.Quantised(h.as_subclass(torch.Tensor).cpu(), h.fp8_meta.amax.cpu(), h.fp8_meta.scale.cpu(), O.E4M3)
         wq = O.quantise_current(w2, O.E4M3)
         assert O.rel_l2(y.cpu(), O.linear_forward(hq, wq)) <= 1e-3
+    # a bias is allowed with an fp8 output: it is added in the epilogue, before the cast (tests/test_gpu_extensions.py)
+    assert FP8Linear(H, I, bias=True, device="cuda", out_dtype=DTypes.FP8E4M3).bias is not None
     with pytest.raises(ValueError):
-        FP8Linear(H, I, bias=True, device="cuda", out_dtype=DTypes.FP8E4M3)
+        FP8Linear(H, I, bias=False, device="cuda", out_dtype=DTypes.KFLOAT16)
     assert "fp8_state.output" in first.state_dict()
 
 
@@ -288,7 +290,7 @@ def test_batch_mixes_fp8_and_plain_outputs_and_rejects_bad_requests():
                                       st) == codes["size, history length or margin out of range"]
     assert nt.lib.ntfp8_amax_finalize(None, 0, 0, state.data_ptr(), None, 0, amax.data_ptr(), None, st) == codes["a required pointer is NULL"]
     torch.cuda.synchronize()
-    assert ctypes.sizeof(nt.GemmDesc) == 112
+    assert ctypes.sizeof(nt.GemmDesc) == 128
 
 
 def test_fp8_output_chain_replayed_as_a_graph_matches_eager():
