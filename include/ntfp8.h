@@ -136,6 +136,19 @@ typedef struct ntfp8_quant_desc {
 } ntfp8_quant_desc;
 int ntfp8_quantize_delayed_batch(const ntfp8_quant_desc* tensors, int count, void* stream);
 
+/* ntfp8_quantize_delayed_batch for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid it).  It has no counterpart in the reference.  The reduction workspaces come
+ * from an array inside the library's device image (NTFP8_STATIC_MAX_TENSORS x NTFP8_WORKSPACE_BYTES = 32 KiB, held
+ * by every GPU the library runs on until the process ends); the `workspace` members of the descriptors are ignored.
+ * count above NTFP8_STATIC_MAX_TENSORS returns NTFP8_ERR_SIZE.  Nothing is allocated or freed, here or in any
+ * routine it calls.  All calls on one GPU share that GPU's array: calls that may overlap in time (different
+ * streams, different threads) race; order them, or use ntfp8_quantize_delayed_batch with workspaces of their own.
+ * The per-device address of the array is resolved at the first call on a device (a host-side look-up plus one
+ * small clearing kernel on `stream`); ntfp8_static_init does that ahead of time for the current device, e.g. before
+ * a graph capture begins. */
+#define NTFP8_STATIC_MAX_TENSORS 16
+int ntfp8_static_init(void* stream);
+int ntfp8_quantize_delayed_batch_static(const ntfp8_quant_desc* tensors, int count, void* stream);
 
 /* out = out_dtype(fp32(fp8) * (1 / *scale)).  Replaces tex.cast_from_fp8
  * (src/nanotron/fp8/tensor.py:74) with meta.inverse_scale (src/nanotron/fp8/meta.py:36-37). */

@@ -18,6 +18,7 @@ E4M3, E5M2 = 0, 1
 F32, F16, BF16 = 0, 1, 2
 OUT_E4M3, OUT_E5M2 = 3, 4  # d_dtype of an fp8 GEMM output
 WORKSPACE_BYTES = 2048
+STATIC_MAX_TENSORS = 16  # tensors per ntfp8_quantize_delayed_batch_static call
 
 TORCH_TO_NT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
@@ -59,6 +60,8 @@ SIGNATURES = {
     "ntfp8_quantize_current": (_i, [_vp, _i, _i64, _i64, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp]),
     "ntfp8_quantize_delayed": (_i, [_vp, _i, _i64, _i64, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "ntfp8_quantize_delayed_batch": (_i, [_c.POINTER(QuantDesc), _i, _vp]),
+    "ntfp8_quantize_delayed_batch_static": (_i, [_c.POINTER(QuantDesc), _i, _vp]),
+    "ntfp8_static_init": (_i, [_vp]),
     "ntfp8_quantize_delayed_dual": (_i, [_vp, _i, _i64, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "ntfp8_te_cast_to_fp8": (_i, [_vp, _i, _i64, _vp, _vp, _vp, _i, _vp, _vp, _vp]),
     "ntfp8_cast_from_fp8": (_i, [_vp, _i, _vp, _i64, _vp, _i, _vp]),

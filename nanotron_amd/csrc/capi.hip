@@ -10,7 +10,8 @@ int run_dequant(const void* in, int fmt, const float* scale, int is_inverse, int
                 hipStream_t st);
 int run_quant_dual(const void* x, int x_dtype, int64_t n, uint8_t* out_e4m3, uint8_t* out_e5m2, Workspace* ws,
                    const ScalarIO& io_e4m3, const ScalarIO& io_e5m2, hipStream_t st);
-
+int static_scratch(void** out, hipStream_t st);
+int run_quant_delayed_batch_static(QuantDesc* q, int count, hipStream_t st);
 int run_transpose(const void* in, int64_t rows, int64_t cols, void* out, hipStream_t st);
 int run_update_scale(const float* amax, const float* old_scale, int fmt, int margin, float* out, int64_t n,
                      hipStream_t st);
@@ -245,6 +246,20 @@ int ntfp8_quantize_delayed_batch(const ntfp8_quant_desc* tensors, int count, voi
     if (rc) return rc;
     return run_quant_delayed_batch(q, count, static_cast<hipStream_t>(stream));
 }
+
+/* BEGIN static-scratch entry points */
+int ntfp8_static_init(void* stream) {
+    void* p = nullptr;
+    return static_scratch(&p, static_cast<hipStream_t>(stream));
+}
+
+int ntfp8_quantize_delayed_batch_static(const ntfp8_quant_desc* tensors, int count, void* stream) {
+    QuantDesc q[NTFP8_STATIC_MAX_TENSORS];
+    const int rc = check_quant_batch(tensors, count, NTFP8_STATIC_MAX_TENSORS, false, q);
+    if (rc) return rc;
+    return run_quant_delayed_batch_static(q, count, static_cast<hipStream_t>(stream));
+}
+/* END static-scratch entry points */
 
 int ntfp8_te_cast_to_fp8(const void* x, int x_dtype, int64_t n, const float* scale, float* amax_inout, float* scale_inv_out,
                          int fmt, void* out, void* workspace, void* stream) {

@@ -752,6 +752,48 @@ int run_quant_dual(const void* x, int x_dtype, int64_t n, uint8_t* out_e4m3, uin
     return check_launch();
 }
 
+// ---------------------------------------------------------------------------------------------
+// Reduction workspaces that live in the library's own device image, for callers that cannot allocate device
+// memory (HIP graph capture, serving loops): one Workspace per tensor of a batched call.  Every GPU the library
+// runs on holds its own copy of the array, at its own address, until the process ends; the name below is only a
+// host-side handle of it, the address comes from hipGetSymbolAddress with that device current.
+static __device__ __align__(256) unsigned char scratch[NTFP8_STATIC_MAX_TENSORS * NTFP8_WORKSPACE_BYTES];
+
+__global__ void fill_zero_kernel(uint32_t* p, int words) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < words) p[i] = 0u;
+}
+
+// Device address of `scratch` on the current device, resolved (and the array cleared, on `st`) at the first call
+// for that device.
+int static_scratch(void** out, hipStream_t st) {
+    static std::atomic<void*> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return NTFP8_ERR_LAUNCH;
+    void* p = cached[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return NTFP8_ERR_LAUNCH;
+        // a loaded image starts zeroed and every kernel leaves its workspace zero; cleared once more here so that
+        // the first user does not depend on the loader
+        constexpr int words = NTFP8_STATIC_MAX_TENSORS * NTFP8_WORKSPACE_BYTES / 4;
+        clear_stale_error();
+        hipLaunchKernelGGL(fill_zero_kernel, dim3((words + 255) / 256), dim3(256), 0, st, static_cast<uint32_t*>(p), words);
+        if (hipGetLastError() != hipSuccess) return NTFP8_ERR_LAUNCH;
+        cached[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return NTFP8_OK;
+}
+
+// run_quant_delayed_batch with the workspaces taken from the static array (count <= NTFP8_STATIC_MAX_TENSORS)
+int run_quant_delayed_batch_static(QuantDesc* q, int count, hipStream_t st) {
+    void* base = nullptr;
+    const int rc = static_scratch(&base, st);
+    if (rc != NTFP8_OK) return rc;
+    for (int i = 0; i < count; ++i) q[i].ws = static_cast<unsigned char*>(base) + (size_t)i * NTFP8_WORKSPACE_BYTES;
+    return run_quant_delayed_batch(q, count, st);
+}
+
 int run_dequant(const void* in, int fmt, const float* scale, int is_inverse, int64_t n, void* out, int out_dtype,
                 hipStream_t st) {
     clear_stale_error();

@@ -268,3 +268,36 @@ def test_batched_quantise_requests_are_validated_before_any_launch():
     assert L.ntfp8_quantize_delayed_batch(shared, 2, None) == -7
     shared = (nt.QuantDesc * 2)(desc(0), desc(1, scale_state=P + 4096))                        # ... or one scaling state
     assert L.ntfp8_quantize_delayed_batch(shared, 2, None) == -7
+
+
+def test_static_scratch_entry_point_rejects_what_it_cannot_hold():
+    """ntfp8_quantize_delayed_batch_static: more tensors than the static array has workspaces for, and every bad
+    argument of the allocating variant, are refused on the host; the `workspace` members are not looked at."""
+    from nanotron_amd import _native as nt
+
+    L = nt.lib
+    P = 0x400000
+    src = open(HEADER).read()
+    assert int(re.search(r"#define NTFP8_STATIC_MAX_TENSORS (\d+)", src).group(1)) == nt.STATIC_MAX_TENSORS
+
+    def desc(k, **kw):
+        d = nt.QuantDesc()
+        base = P + k * (1 << 20)
+        d.x, d.x_dtype, d.fmt, d.margin, d.history_len, d.rows, d.cols = base, 2, 0, 0, 16, 4, 4
+        d.scale_state, d.amax_history, d.amax_out, d.out = base + 4096, base + 4100, base + 8192, base + 12288
+        for name, v in kw.items():
+            setattr(d, name, v)
+        return d
+
+    n = nt.STATIC_MAX_TENSORS + 1
+    many = (nt.QuantDesc * n)(*[desc(k) for k in range(n)])
+    assert L.ntfp8_quantize_delayed_batch_static(many, n, None) == -3
+    assert "size" in nt.strerror(-3)
+    one = lambda d: (nt.QuantDesc * 1)(d)
+    assert L.ntfp8_quantize_delayed_batch_static(None, 1, None) == -1
+    assert L.ntfp8_quantize_delayed_batch_static(one(desc(0)), 0, None) == -3
+    assert L.ntfp8_quantize_delayed_batch_static(one(desc(0, out=None)), 1, None) == -1
+    assert L.ntfp8_quantize_delayed_batch_static(one(desc(0, rows=0)), 1, None) == -3
+    assert L.ntfp8_quantize_delayed_batch_static(one(desc(0, out=P + 8)), 1, None) == -7
+    two = (nt.QuantDesc * 2)(desc(0), desc(1, amax_out=P + 8192))
+    assert L.ntfp8_quantize_delayed_batch_static(two, 2, None) == -7
