@@ -6,11 +6,14 @@
 Default workload ("linear"): the Llama-3-8B decoder-block linears of the benchmark configuration,
 forward + backward with delayed scaling (history 16, margin 0) at 4096 tokens:
 QKV 4096->6144, O 4096->4096, gate 4096->14336, up 4096->14336, down 14336->4096.
-One step = for every linear: re-quantise the weight (e4m3, + transpose), quantise the activation
-(e4m3, + transpose), forward GEMM (bf16 out), quantise the output gradient (e5m2, + transpose),
-dgrad GEMM (bf16 out), wgrad GEMM (fp32 out).  All inputs are resident in HBM before the timed
-region.  value = GEMM FLOPs of the step (6*M*N*K per linear) / wall time of the step, so the
-quantisation passes are inside the time but contribute no FLOPs.
+One step = the bf16 master weights take the step's (perturbed) values and their fp8 copies are refreshed
+(e4m3, one batched call); then for every linear: quantise the step's activation (e4m3), forward GEMM (bf16 out),
+quantise the step's output gradient (e5m2, with its transposed copy), dgrad GEMM (bf16 out) and wgrad GEMM (fp32
+out) in one batched call.  Inputs of ten steps (fresh seeded X / dY, perturbed weights) are resident in HBM before
+the timed region and are walked round robin.  Before anything is timed, steps 0 and 1 are compared with the CPU
+oracle (bit-exact amax / scales / histories / fp8 bytes, GEMM results within rel-L2 1e-3); a mismatch ends the run
+without a line.  value = GEMM FLOPs of the step (6*M*N*K per linear) / wall time of the step, so the quantisation
+passes are inside the time but contribute no FLOPs.
 
 Workload "quant": benchmark configuration 2, the fused amax + history roll + scale update +
 saturating cast on bf16 [4096,4096], e4m3 and e5m2 alternating, 8 rotating input buffers.
@@ -31,15 +34,13 @@ if ROOT not in sys.path:
 
 PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA peak
 PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E peak
-# HBM-side traffic measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (one counter per run, KiB per dispatch
-# scaled by what the same counter reads for a 128 MiB copy: x2.0 for FETCH_SIZE, x1.0 for WRITE_SIZE); the figures
-# and the commands are in profiles/hbm_traffic_counters.txt.  Bytes, summed over the GEMM launches of one step /
-# for one launch of the fused quantise kernel on the [4096,4096] bf16 tensor.
-GEMM_TRAFFIC_PER_STEP = {"fetch": 4133.3e6, "write": 1478.7e6}
-QUANT_TRAFFIC_PER_LAUNCH = {"fetch": 33.67e6, "write": 16.79e6}
+# HBM-side traffic is not measurable from inside this process: it comes from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs of this same script, whose summary (figures, commands, the commit and flags they were taken at) is the text
+# file below.  Its "bench-readable" block is parsed here and handed on with its provenance.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_counters.txt")
 
 TOKENS = 4096
-LINEARS = [  # name, in_features (K), out_features (N)
+LINEARS = [  # name, in_features (K), out_features (N): benchmark configuration 5 (the parity test uses the same list)
     ("qkv", 4096, 6144),
     ("o", 4096, 4096),
     ("gate", 4096, 14336),
@@ -62,7 +63,48 @@ def parse():
                         "those (the reference's way) instead of letting the GEMM read the tensors as they are")
     p.add_argument("--kernel-reps", type=int, default=0,
                    help="also time each GEMM shape in isolation with this many back-to-back launches (0 = skip)")
+    p.add_argument("--fp8-activations", action="store_true",
+                   help="every linear returns its output as an e4m3 FP8Tensor quantised in the GEMM epilogue "
+                        "(no bf16 activation is written); not the headline configuration")
+    p.add_argument("--no-verify", action="store_true",
+                   help="skip the correctness gate (profiling runs only: the line then says verified = false)")
     return p.parse_args()
+
+
+def flags_of(args):
+    """The switches that change which kernels a step launches, as one string (recorded next to counter figures)."""
+    on = [n for n in ("weight_stream", "transposed_copies", "fp8_activations") if getattr(args, n)]
+    return "default" if not on else ",".join(on)
+
+
+def read_traffic(args):
+    """{"gemm": bytes per step | None, "quant": bytes per launch | None, "source": {...}} from the bench-readable
+    block of the counter summary under profiles/.  A figure taken with other flags than this run's is not used."""
+    out = {"gemm": None, "quant": None, "source": {"file": os.path.relpath(TRAFFIC_FILE, ROOT)}}
+    try:
+        text = open(TRAFFIC_FILE).read()
+    except OSError:
+        out["source"]["note"] = "file not found"
+        return out
+    kv = {}
+    block = False
+    for line in text.splitlines():
+        if line.startswith("[bench-readable]"):
+            block = True
+            continue
+        if block and "=" in line:
+            k, v = line.split("=", 1)
+            kv[k.strip()] = v.strip()
+    out["source"].update({"commit": kv.get("commit"), "flags": kv.get("flags"), "workload": kv.get("workload")})
+    if kv.get("flags") != flags_of(args):
+        out["source"]["note"] = f"counters were taken with flags '{kv.get('flags')}', this run uses '{flags_of(args)}': not used"
+        return out
+    try:
+        out["gemm"] = float(kv["gemm_fetch_bytes_per_step"]) + float(kv["gemm_write_bytes_per_step"])
+        out["quant"] = float(kv["quant_fetch_bytes_per_launch"]) + float(kv["quant_write_bytes_per_launch"])
+    except (KeyError, ValueError):
+        out["source"]["note"] = "bench-readable block incomplete"
+    return out
 
 
 def event_time_ms(fn, reps, warm=3):
@@ -82,35 +124,78 @@ def event_time_ms(fn, reps, warm=3):
 
 
 # ------------------------------------------------------------------------------------ linear workload
-def build_linears(device):
+def build_linears(device, nsets, fp8_out=False):
+    """The five linears, and `nsets` steps' worth of inputs resident in HBM: per step and layer a fresh seeded X and
+    dY (generated on the CPU, as the oracle sees them) and a version of the bf16 master weight, each version the
+    previous one plus a seeded perturbation: the stand-in for an optimizer update, so that the weight role's amax
+    history moves.  A step swaps the layer's parameter for that step's version (a pointer swap, no device work)."""
     import torch
 
     from nanotron_amd.fp8 import DTypes, FP8Linear, FP8Parameter
+    from oracle import step_check as C
 
-    g = torch.Generator(device="cpu").manual_seed(1234 + 500)
-    mods, xs, gys = [], [], []
-    for name, K, N in LINEARS:
-        lin = FP8Linear(K, N, bias=False, device=device, out_dtype=torch.bfloat16, delayed_scaling=True,
-                        amax_history_len=16, margin=0)
-        # bf16 master weights ~N(0, 0.02), re-quantised (delayed scaling) every step
-        w = (torch.randn(N, K, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16)
-        lin.weight = FP8Parameter(w.to(device), DTypes.FP8E4M3)
+    mods, cpu = [], []
+    sets = [{"x": [], "gy": [], "w": []} for _ in range(nsets)]
+    for i, (name, K, N) in enumerate(LINEARS):
+        lin = FP8Linear(K, N, bias=False, device=device, out_dtype=DTypes.FP8E4M3 if fp8_out else torch.bfloat16,
+                        delayed_scaling=True, amax_history_len=16, margin=0)
+        w = C.initial_weight(i, K, N)
+        per_step = []
+        for s_ in range(nsets):
+            w = C.perturbed_weight(w, s_, i)
+            x, gy = C.step_inputs(s_, i, K, N)
+            sets[s_]["w"].append(FP8Parameter(w.to(device), DTypes.FP8E4M3))
+            sets[s_]["x"].append(x.to(device).requires_grad_(True))
+            sets[s_]["gy"].append(gy.to(device))
+            if s_ < 2:   # what the correctness gate compares with
+                per_step.append((x, w, gy))
+        lin.weight = sets[0]["w"][i]
         mods.append(lin)
-        xs.append((torch.randn(TOKENS, K, generator=g, dtype=torch.float32)).to(torch.bfloat16).to(device))
-        gys.append((torch.randn(TOKENS, N, generator=g, dtype=torch.float32) * 1e-3).to(torch.bfloat16).to(device))
-    return mods, xs, gys
+        cpu.append(per_step)
+    return mods, sets, cpu
 
 
-def linear_step(mods, xs, gys, wstream=None):
+def linear_step(mods, sets, index, wstream=None, fp8_out=False, check=None):
+    """One step: the master weights take this step's values, the fp8 copies of all weights are refreshed (one batched
+    library call on the compute stream, or per layer on a second stream), then forward + backward of every linear.
+    `check(i, lin, x, y, saved_input)` is called after each layer by the correctness gate."""
     from nanotron_amd.fp8.optim import requantize_fp8_weights
 
-    # the fp8 copies of all weights are refreshed from their masters first, as after an optimizer step: one batched
-    # library call on the compute stream, or (--weight-stream) per-layer calls on a second stream
+    cur = sets[index % len(sets)]
+    for lin, w in zip(mods, cur["w"]):
+        lin.weight = w
     requantize_fp8_weights(mods, stream=wstream)
-    for lin, x, gy in zip(mods, xs, gys):
+    for i, (lin, x, gy) in enumerate(zip(mods, cur["x"], cur["gy"])):
         x.grad = None
         y = lin(x)
-        y.backward(gy)
+        saved = y.grad_fn.saved_tensors[0] if check is not None and y.grad_fn is not None else None
+        if fp8_out:
+            y._grad_handle.backward(gy)   # the gradient of an fp8 output travels through its handle
+        else:
+            y.backward(gy)
+        if check is not None:
+            check(i, lin, x, y, saved)
+
+
+def verify_steps(mods, sets, cpu, wstream):
+    """The correctness gate: steps 0 and 1 of the workload (the first quantises with current scaling, the second
+    runs the fused delayed-scaling kernels that the timed steps run) are compared layer by layer with the CPU oracle:
+    amax, scales, amax histories and fp8 bytes bit for bit, Y / dX / dW on sampled rows within rel-L2 1e-3.
+    Raises AssertionError on the first difference.  Returns the largest rel-L2 seen per GEMM kind."""
+    from oracle import step_check as C
+
+    assert C.LINEARS == LINEARS and C.TOKENS == TOKENS
+    refs = C.new_reference_state()
+    worst = {"fwd": 0.0, "dgrad": 0.0, "wgrad": 0.0}
+    for step in range(2):
+        def check(i, lin, x, y, saved):
+            xc, wc, gc = cpu[i][step]
+            errs = C.check_layer(f"step {step} {LINEARS[i][0]}", lin, refs[i], xc, wc, gc, y.detach(), x.grad,
+                                 lin.weight.main_grad, saved, step, i)
+            for k, v in errs.items():
+                worst[k] = max(worst[k], v)
+        linear_step(mods, sets, step, wstream, check=check)
+    return {k: float(f"{v:.3e}") for k, v in worst.items()}
 
 
 def gemm_algorithmic_bytes():
@@ -131,7 +216,7 @@ def gemm_in_step_timing(step, first_index, steps):
 
     from nanotron_amd.fp8 import kernel as K
 
-    orig_one, orig_batch = K._gemm_nt, K._gemm_nt_batch
+    orig_one, orig_batch, orig_fp8 = K._gemm_nt, K._gemm_nt_batch, K._gemm_nt_fp8
     log = []
 
     def bracket(fn, shapes):
@@ -143,21 +228,24 @@ def gemm_in_step_timing(step, first_index, steps):
         log.append((shapes, e0, e1))
         return out
 
-    def timed_one(a, b, out_dtype, accumulate_into):
-        return bracket(lambda: orig_one(a, b, out_dtype, accumulate_into), [(a.shape[0], b.shape[0], a.shape[1])])
+    def timed_one(a, b, out_dtype, accumulate_into, bias=None):
+        return bracket(lambda: orig_one(a, b, out_dtype, accumulate_into, bias), [(a.shape[0], b.shape[0], a.shape[1])])
+
+    def timed_fp8(a, b, dtype, state, with_transpose, bias=None):
+        return bracket(lambda: orig_fp8(a, b, dtype, state, with_transpose, bias), [(a.shape[0], b.shape[0], a.shape[1])])
 
     def timed_batch(problems):
         # a fifth element marks a B operand handed over as its [K, N] transpose
         return bracket(lambda: orig_batch(problems),
                        [(p[0].shape[0], p[1].shape[1 if len(p) > 4 and p[4] else 0], p[0].shape[1]) for p in problems])
 
-    K._gemm_nt, K._gemm_nt_batch = timed_one, timed_batch
+    K._gemm_nt, K._gemm_nt_batch, K._gemm_nt_fp8 = timed_one, timed_batch, timed_fp8
     try:
         for i in range(steps):
             step(first_index + i)
         torch.cuda.synchronize()
     finally:
-        K._gemm_nt, K._gemm_nt_batch = orig_one, orig_batch
+        K._gemm_nt, K._gemm_nt_batch, K._gemm_nt_fp8 = orig_one, orig_batch, orig_fp8
     per_step = len(log) // steps
     names = [f"{n}.{t}" for n, _, _ in LINEARS for t in ("fwd", "dgrad+wgrad")]
     assert per_step == len(names), (per_step, len(names))
@@ -173,7 +261,7 @@ def gemm_in_step_timing(step, first_index, steps):
     return total_flops, total_ms, per_call
 
 
-def gemm_isolated_timing(mods, xs, gys, reps):
+def gemm_isolated_timing(mods, sets, reps):
     """Back-to-back launches of each GEMM of the step on fixed operands (which then sit in the 256 MB
     memory-side cache): an upper bound on what the kernel does in the step, reported for comparison."""
     import torch
@@ -182,7 +270,7 @@ def gemm_isolated_timing(mods, xs, gys, reps):
     from nanotron_amd.fp8.kernel import _gemm_nt
 
     per_shape = []
-    for (name, K, N), lin, x, gy in zip(LINEARS, mods, xs, gys):
+    for (name, K, N), lin, x, gy in zip(LINEARS, mods, sets[0]["x"], sets[0]["gy"]):
         xq = FP8Tensor(x.detach(), DTypes.FP8E4M3, with_transpose=True)
         gq = FP8Tensor(gy, DTypes.FP8E5M2, with_transpose=True)
         wq = lin.weight.data
@@ -226,7 +314,32 @@ def cpu_baseline_linear():
         n += 1
     dt = (time.perf_counter() - t0) / n
     return {"value": round(6.0 * M * N * K / dt / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
-            "kind": "port", "sample": f"O projection 4096x4096x4096 fwd+bwd (quantise X,W,dY + 3 fp32 GEMMs), {n} runs"}
+            "kind": "port", "sample": f"O projection 4096x4096x4096 fwd+bwd (quantise X,W,dY + 3 fp32 GEMMs), {n} runs",
+            "reference_cpu_path": cpu_reference_path_config1()}
+
+
+def cpu_reference_path_config1():
+    """What the reference itself executes when the tensors are on the CPU: plain `F.linear` in the tensors' own
+    precision, no FP8 at all (src/nanotron/fp8/linear.py:53-54), on benchmark configuration 1 (X [2048,1024] ~N(0,1),
+    W [1024,1024] ~N(0,0.02)), fp32 as FP8Linear(device="cpu") creates its weight.  Forward only, as the configuration."""
+    import torch
+    import torch.nn.functional as F
+
+    from oracle import fp8_oracle as O
+
+    x = O.normal_tensor(1234 + 100, (2048, 1024), 1.0, torch.float32)
+    w = O.normal_tensor(1234 + 101, (1024, 1024), 0.02, torch.float32)
+    for _ in range(3):
+        F.linear(x, w)
+    times = []
+    t_end = time.perf_counter() + 3.0
+    while len(times) < 5 or time.perf_counter() < t_end:
+        t0 = time.perf_counter()
+        F.linear(x, w)
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {"value": round(2.0 * 2048 * 1024 * 1024 / med / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "reference", "sample": f"config 1: fp32 F.linear X[2048,1024] . W[1024,1024]^T on the CPU, median of {len(times)} runs"}
 
 
 # ------------------------------------------------------------------------------------ quant workload
@@ -258,7 +371,8 @@ def quant_kernel_ms(bufs, states, reps):
     from nanotron_amd.fp8 import DTypes
 
     dev = bufs[0].device
-    out = [torch.empty(4096 * 4096, dtype=torch.uint8, device=dev) for _ in range(len(bufs))]
+    rows, cols = bufs[0].shape
+    out = [torch.empty(rows * cols, dtype=torch.uint8, device=dev) for _ in range(len(bufs))]
     sc = torch.zeros(2, dtype=torch.float32, device=dev)
     ws = nt.workspace(dev)
     st = nt.stream_ptr(dev)
@@ -270,13 +384,85 @@ def quant_kernel_ms(bufs, states, reps):
         def fn():
             i = k[0] % len(bufs)
             k[0] += 1
-            nt.check(nt.lib.ntfp8_quantize_delayed(bufs[i].data_ptr(), nt.BF16, 4096, 4096, fmt, 0,
+            nt.check(nt.lib.ntfp8_quantize_delayed(bufs[i].data_ptr(), nt.BF16, rows, cols, fmt, 0,
                                                    state.scale.data_ptr(), state.amax_history.data_ptr(), 16,
                                                    sc[0:].data_ptr(), sc[1:].data_ptr(), out[i].data_ptr(), None,
                                                    ws.data_ptr(), st), "quantize_delayed")
 
         res[dt.name] = event_time_ms(fn, reps, warm=8)
     return res
+
+
+def quant_dual_kernel_ms(bufs, states, reps):
+    """Average duration of the kernel that produces both formats from one pass over the tensor."""
+    import torch
+
+    from nanotron_amd import _native as nt
+    from nanotron_amd.fp8 import DTypes
+
+    dev = bufs[0].device
+    n = bufs[0].numel()
+    out4 = [torch.empty(n, dtype=torch.uint8, device=dev) for _ in range(len(bufs))]
+    out5 = [torch.empty(n, dtype=torch.uint8, device=dev) for _ in range(len(bufs))]
+    sc = torch.zeros(3, dtype=torch.float32, device=dev)
+    ws = nt.workspace(dev)
+    st = nt.stream_ptr(dev)
+    s4, s5 = states[DTypes.FP8E4M3], states[DTypes.FP8E5M2]
+    k = [0]
+
+    def fn():
+        i = k[0] % len(bufs)
+        k[0] += 1
+        nt.check(nt.lib.ntfp8_quantize_delayed_dual(bufs[i].data_ptr(), nt.BF16, n, 0, s4.scale.data_ptr(),
+                                                    s4.amax_history.data_ptr(), s5.scale.data_ptr(), s5.amax_history.data_ptr(),
+                                                    16, sc.data_ptr(), sc.data_ptr() + 4, sc.data_ptr() + 8,
+                                                    out4[i].data_ptr(), out5[i].data_ptr(), ws.data_ptr(), st), "quantize_delayed_dual")
+
+    return event_time_ms(fn, reps, warm=8)
+
+
+def quant_report(device, traffic):
+    """The `quant` object of the JSON line: the fused quantise kernel on benchmark configuration 2 (bf16 [4096,4096],
+    8 rotating buffers so that the input does not sit in the memory-side cache), the both-formats-in-one-pass kernel on
+    the same tensor, and the single-format kernel on the largest tensors of the step, where the launch ramp and the
+    end-of-kernel reduction weigh less."""
+    import torch
+
+    from nanotron_amd.fp8 import DelayedScaling, DTypes
+
+    bufs, states = build_quant(device)
+    for i in range(2):   # both roles hold a scale from here on
+        quant_step(bufs, states, i)
+    qms = quant_kernel_ms(bufs, states, 64)
+    qb = 3.0 * 4096 * 4096
+    q_avg = sum(qms.values()) / len(qms)
+    dual_ms = quant_dual_kernel_ms(bufs, states, 64)
+    rep = {"metric": "amax+quant GB/s", "value": round(qb / (q_avg * 1e-3) / 1e9, 1), "unit": "GB/s",
+           "workload": "bf16 [4096,4096] fused amax+roll+scale+cast, 8 rotating buffers",
+           "ms": {k: round(v, 5) for k, v in qms.items()},
+           "roofline": {"bound": "hbm", "achieved": round(qb / (q_avg * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                        "frac": round(qb / (q_avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4), "traffic": traffic["quant"],
+                        "algorithmic_bytes": qb, "kernel": "quant_flat_kernel"},
+           "both_formats_one_pass": {"ms": round(dual_ms, 5), "algorithmic_bytes": 4.0 * 4096 * 4096,
+                                     "GBps": round(4.0 * 4096 * 4096 / (dual_ms * 1e-3) / 1e9, 1),
+                                     "frac": round(4.0 * 4096 * 4096 / (dual_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+                                     "kernel": "quant_flat_dual_kernel"}}
+    del bufs
+    large = {}
+    g = torch.Generator(device=device).manual_seed(99)
+    for shape in ((4096, 14336), (14336, 4096)):
+        lb = [torch.randn(shape, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16) for _ in range(4)]
+        st = {DTypes.FP8E4M3: DelayedScaling(DTypes.FP8E4M3, 16, 0, device), DTypes.FP8E5M2: DelayedScaling(DTypes.FP8E5M2, 16, 0, device)}
+        for i in range(2):
+            quant_step(lb, st, i)
+        ms = quant_kernel_ms(lb, st, 32)
+        avg = sum(ms.values()) / len(ms)
+        nbytes = 3.0 * shape[0] * shape[1]
+        large[f"{shape[0]}x{shape[1]}"] = {"ms": round(avg, 5), "GBps": round(nbytes / (avg * 1e-3) / 1e9, 1),
+                                            "frac": round(nbytes / (avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)}
+        del lb
+    rep["large_tensors"] = large
+    return rep
 
 
 def cpu_baseline_quant():
@@ -360,23 +546,37 @@ def main():
     if args.workload == "probe":
         probe(device)
         return
+    traffic = read_traffic(args)
+    verified = None
     if args.workload == "linear":
-        mods, xs, gys = build_linears(device)
-        xs = [x.requires_grad_(True) for x in xs]
+        # ten steps' worth of inputs (benchmark configuration 5), fewer if the run is shorter than that
+        nsets = max(2, min(10, args.warmup + 2 * args.steps))
+        mods, sets, cpu = build_linears(device, nsets, fp8_out=args.fp8_activations)
         wstream = torch.cuda.Stream(device=device) if args.weight_stream else None
-        step = lambda i: linear_step(mods, xs, gys, wstream)
+        step = lambda i: linear_step(mods, sets, i, wstream, fp8_out=args.fp8_activations)
         flops_step = sum(6.0 * TOKENS * N * K for _, K, N in LINEARS)
+        first = 0
+        if not args.no_verify and not args.fp8_activations:
+            # correctness gate: no line is printed for a step that does not match the oracle
+            try:
+                verified = verify_steps(mods, sets, cpu, wstream)
+            except AssertionError as e:
+                print(f"bench.py: the workload's results differ from the CPU oracle, nothing measured: {e}", file=sys.stderr)
+                sys.exit(1)
+            first = 2
+        del cpu
     else:
         bufs, states = build_quant(device)
         step = lambda i: quant_step(bufs, states, i)
         bytes_step = 2 * 3.0 * 4096 * 4096
+        first = 0
 
     for i in range(args.warmup):
-        step(i)
+        step(first + i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(args.warmup + i)
+        step(first + args.warmup + i)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
@@ -387,36 +587,33 @@ def main():
     }
     if args.workload == "linear":
         value = flops_step / (ms_per_step * 1e-3) / 1e12
-        gf, gms, per_call = gemm_in_step_timing(step, args.warmup + args.steps, args.steps)
+        gf, gms, per_call = gemm_in_step_timing(step, first + args.warmup + args.steps, args.steps)
         achieved = gf / (gms * 1e-3) / 1e12
+        acts = "e4m3 activations out of the GEMM epilogue" if args.fp8_activations else "bf16 activations"
         out.update({
             "metric": "FP8Linear fwd+bwd TFLOP/s", "value": round(value, 2), "unit": "TFLOP/s", "dtype": "fp8",
-            "config": {"workload": "llama3-8b decoder-block linears fwd+bwd, 4096 tokens, bf16 activations and weights, delayed scaling hist 16",
+            "config": {"workload": f"llama3-8b decoder-block linears fwd+bwd, 4096 tokens, {acts}, bf16 master weights, "
+                                   "delayed scaling hist 16, fresh seeded X/dY and perturbed weights every step",
                        "weight_requantisation": "second stream, per layer" if args.weight_stream else "compute stream, one batched call per step",
-                       "tokens": TOKENS, "linears": [f"{n}:{k}->{o}" for n, k, o in LINEARS],
-                       "flops_per_step": flops_step, "pct_fp8_peak": round(100 * value / PEAK_FP8_TFLOPS, 2)},
+                       "tokens": TOKENS, "linears": [f"{n}:{k}->{o}" for n, k, o in LINEARS], "input_sets": len(sets),
+                       "flags": flags_of(args), "flops_per_step": flops_step, "pct_fp8_peak": round(100 * value / PEAK_FP8_TFLOPS, 2)},
+            "verified": ({"against": "CPU oracle, steps 0 and 1: amax / scales / histories / fp8 bytes bit-exact, "
+                                     "Y / dX / dW on sampled rows", "worst_rel_l2": verified} if verified is not None else False),
             "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(achieved / PEAK_FP8_TFLOPS, 4),
-                         "traffic": GEMM_TRAFFIC_PER_STEP["fetch"] + GEMM_TRAFFIC_PER_STEP["write"],
+                         "traffic": traffic["gemm"],
                          "traffic_unit": "bytes per step, all GEMM launches (fetch + write counters)",
+                         "traffic_source": traffic["source"],
                          "algorithmic_bytes": gemm_algorithmic_bytes(),
                          "kernel": "gemm_nt_big_kernel", "timing": "HIP events around every GEMM call inside the step",
                          "gemm_ms_per_step": round(gms, 4), "calls": per_call},
         })
         if args.kernel_reps > 0:
-            out["roofline"]["isolated"] = gemm_isolated_timing(mods, xs, gys, args.kernel_reps)
+            out["roofline"]["isolated"] = gemm_isolated_timing(mods, sets, args.kernel_reps)
+        del mods, sets
+        torch.cuda.empty_cache()
         # secondary figure of the metric: the fused quantise kernel on configuration 2
-        bufs, states = build_quant(device)
-        qms = quant_kernel_ms(bufs, states, 64)
-        qb = 3.0 * 4096 * 4096
-        q_avg = sum(qms.values()) / len(qms)
-        out["quant"] = {"metric": "amax+quant GB/s", "value": round(qb / (q_avg * 1e-3) / 1e9, 1), "unit": "GB/s",
-                        "workload": "bf16 [4096,4096] fused amax+roll+scale+cast, 8 rotating buffers",
-                        "ms": {k: round(v, 5) for k, v in qms.items()},
-                        "roofline": {"bound": "hbm", "achieved": round(qb / (q_avg * 1e-3) / 1e9, 1),
-                                     "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                                     "frac": round(qb / (q_avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
-                                     "traffic": sum(QUANT_TRAFFIC_PER_LAUNCH.values()), "algorithmic_bytes": qb}}
+        out["quant"] = quant_report(device, traffic)
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_baseline_linear()
     else:
@@ -430,7 +627,7 @@ def main():
                        "bytes_per_step": bytes_step, "pct_hbm_peak": round(100 * value / PEAK_HBM_GBPS, 2)},
             "roofline": {"bound": "hbm", "achieved": round(qb / (q_avg * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBPS,
                          "unit": "GB/s", "frac": round(qb / (q_avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
-                         "traffic": sum(QUANT_TRAFFIC_PER_LAUNCH.values()), "algorithmic_bytes": qb,
+                         "traffic": traffic["quant"], "traffic_source": traffic["source"], "algorithmic_bytes": qb,
                          "kernel": "quant_flat_kernel", "ms": {k: round(v, 5) for k, v in qms.items()}},
         })
         if not args.no_cpu_baseline:
