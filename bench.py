@@ -61,6 +61,9 @@ def parse():
     p.add_argument("--transposed-copies", action="store_true",
                    help="quantise weights and inputs together with transposed copies and run the backward GEMMs on "
                         "those (the reference's way) instead of letting the GEMM read the tensors as they are")
+    p.add_argument("--grad-transposed-copy", action="store_true",
+                   help="quantise the output gradient together with its transposed copy and run wgrad on that (the "
+                        "reference's way, kernel.py:44) instead of letting the GEMM read dY as it is")
     p.add_argument("--kernel-reps", type=int, default=0,
                    help="also time each GEMM shape in isolation with this many back-to-back launches (0 = skip)")
     p.add_argument("--fp8-activations", action="store_true",
@@ -73,7 +76,7 @@ def parse():
 
 def flags_of(args):
     """The switches that change which kernels a step launches, as one string (recorded next to counter figures)."""
-    on = [n for n in ("weight_stream", "transposed_copies", "fp8_activations") if getattr(args, n)]
+    on = [n for n in ("weight_stream", "transposed_copies", "grad_transposed_copy", "fp8_activations") if getattr(args, n)]
     return "default" if not on else ",".join(on)
 
 
@@ -235,9 +238,12 @@ def gemm_in_step_timing(step, first_index, steps):
         return bracket(lambda: orig_fp8(a, b, dtype, state, with_transpose, bias), [(a.shape[0], b.shape[0], a.shape[1])])
 
     def timed_batch(problems):
-        # a fifth element marks a B operand handed over as its [K, N] transpose
-        return bracket(lambda: orig_batch(problems),
-                       [(p[0].shape[0], p[1].shape[1 if len(p) > 4 and p[4] else 0], p[0].shape[1]) for p in problems])
+        # elements 5 and 7 of a problem mark operands handed over as their transposes ([K, N] / [K, M])
+        def mnk(p):
+            bt = len(p) > 4 and p[4]
+            at = len(p) > 6 and p[6]
+            return (p[0].shape[1 if at else 0], p[1].shape[1 if bt else 0], p[0].shape[0 if at else 1])
+        return bracket(lambda: orig_batch(problems), [mnk(p) for p in problems])
 
     K._gemm_nt, K._gemm_nt_batch, K._gemm_nt_fp8 = timed_one, timed_batch, timed_fp8
     try:
@@ -542,6 +548,10 @@ def main():
         import nanotron_amd.fp8.kernel as K
 
         K.READ_B_TRANSPOSED = False
+    if args.grad_transposed_copy:
+        import nanotron_amd.fp8.kernel as K
+
+        K.READ_A_TRANSPOSED = False
 
     if args.workload == "probe":
         probe(device)

@@ -208,6 +208,12 @@ typedef struct ntfp8_gemm_desc {
     /* != 0: scale_a and scale_b point to INVERSE scales, the form tex.te_gemm is handed
      * (meta.inverse_scale, src/nanotron/fp8/kernel.py:48,52): the sum is multiplied by them, not divided. */
     int scales_are_inverse;
+    /* != 0: A points to the [K, M] row-major bytes of A's transpose.  The wgrad of a linear layer,
+     * dW = dY^T . X (src/nanotron/fp8/linear.py:107-109), reduces over the rows of both its operands: with
+     * a_transposed and b_transposed set it reads dY[tokens, out] and X[tokens, in] as they are, where the reference
+     * transposes both first (src/nanotron/fp8/kernel.py:43-44).  Only together with b_transposed, under its
+     * conditions, and M a multiple of 16; anything else returns NTFP8_ERR_UNSUPPORTED. */
+    int a_transposed;
 } ntfp8_gemm_desc;
 /* A call that returns an error has launched nothing: every problem is validated, and matched to a kernel, before
  * the first launch. */

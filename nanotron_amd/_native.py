@@ -39,7 +39,7 @@ class GemmDesc(ctypes.Structure):
                 ("M", _i64), ("N", _i64), ("K", _i64),
                 ("fmt_a", _i), ("fmt_b", _i), ("d_dtype", _i), ("accumulate", _i),
                 ("scale_d", _vp), ("D_t", _vp), ("amax_workspace", _vp), ("b_transposed", _i),
-                ("bias", _vp), ("bias_dtype", _i), ("scales_are_inverse", _i)]
+                ("bias", _vp), ("bias_dtype", _i), ("scales_are_inverse", _i), ("a_transposed", _i)]
 
 
 class QuantDesc(ctypes.Structure):

@@ -86,7 +86,8 @@ int check_gemm(const ntfp8_gemm_desc& p, GemmDesc* g) {
     }
     *g = GemmDesc{p.A, p.fmt_a, p.scale_a, p.B, p.fmt_b, p.scale_b, p.D, p.d_dtype, (int)M, (int)N, (int)K, p.accumulate ? 1 : 0,
                   nullptr, nullptr, nullptr, p.b_transposed ? 1 : 0, p.bias, p.bias ? p.bias_dtype : NTFP8_F32,
-                  p.scales_are_inverse ? 1 : 0};
+                  p.scales_are_inverse ? 1 : 0, p.a_transposed ? 1 : 0};
+    if (p.a_transposed && !p.b_transposed) return NTFP8_ERR_UNSUPPORTED;
     if (p.b_transposed && fp8_out) return NTFP8_ERR_UNSUPPORTED;
     if (fp8_out) {
         if (!is_aligned(p.scale_d, 4) || (p.amax_workspace && !is_aligned(p.amax_workspace, 4))) return NTFP8_ERR_ALIGN;
@@ -343,7 +344,7 @@ int ntfp8_gemm(const void* A, int fmt_a, const float* scale_a, const void* B, in
                int d_dtype, int64_t M, int64_t N, int64_t K, int accumulate, void* stream) {
     if (is_fp8_out(d_dtype)) return NTFP8_ERR_UNSUPPORTED;   // fp8 outputs carry more arguments: ntfp8_gemm_batch
     const ntfp8_gemm_desc p = {A, scale_a, B, scale_b, D, M, N, K, fmt_a, fmt_b, d_dtype, accumulate, nullptr, nullptr, nullptr, 0,
-                               nullptr, NTFP8_F32, 0};
+                               nullptr, NTFP8_F32, 0, 0};
     GemmDesc g;
     const int rc = check_gemm(p, &g);
     if (rc) return rc;

@@ -165,6 +165,7 @@ struct GemmDesc {
     const void* bias;
     int bias_dtype;
     int scale_inv;   // scale_a / scale_b point to inverse scales (what tex.te_gemm receives): multiplied, not divided by
+    int ta;          // A is given as [K, M] row-major (its transpose); only together with tb
 };
 
 __host__ __device__ inline bool is_fp8_out(int d_dtype) { return d_dtype == NTFP8_OUT_E4M3 || d_dtype == NTFP8_OUT_E5M2; }

@@ -180,7 +180,9 @@ static int path_of(const GemmDesc& g) {
     const bool fp8_ok = !is_fp8_out(g.d_dtype) ||
                         (g.N % 16 == 0 && g.M % 4 == 0 && (int64_t)g.M * g.N < (1LL << 32) - 16 &&
                          (reinterpret_cast<uintptr_t>(g.Dt) & 15) == 0);
-    // a B operand given as [K, N] is loaded in 16-byte pieces of its rows; only the big kernel reads it
+    // an operand given as its transpose, [K, N] or [K, M], is loaded in 16-byte pieces of its rows; only the big
+    // kernel reads it, and a transposed A only next to a transposed B (the wgrad form)
+    if (g.ta && (!g.tb || g.M % 16 != 0)) return kPathNone;
     if (g.tb) return (g.N % 16 == 0 && fits32 && worth && !is_fp8_out(g.d_dtype)) ? kPathBig : kPathNone;
     return (fits32 && worth && fp8_ok) ? kPathBig : kPathSmall;
 }
@@ -219,6 +221,7 @@ static int launch_big(const GemmDesc* const* g, int n, hipStream_t st) {
         p.accumulate = d.accumulate;
         p.fp8 = Fp8Out{d.sd, static_cast<uint8_t*>(d.Dt), static_cast<Workspace*>(d.ws)};
         p.ex = GemmExtras{d.bias, d.bias_dtype, d.scale_inv};
+        p.at = d.ta;
         tiles += p.tiles_m * p.tiles_n;
     }
     const int rem = tiles % cu_count();

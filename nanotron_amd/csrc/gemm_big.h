@@ -233,6 +233,7 @@ struct BigProblem {
     int accumulate;         // fp32 outputs only: D += result
     Fp8Out fp8;             // fp8 outputs only
     GemmExtras ex;          // bias, inverse-scale flag
+    int at;                 // A is given as [K, M] row-major (its transpose); kBT launches only
 };
 constexpr int kBigMaxProblems = 4;
 struct BigLaunch {
@@ -323,17 +324,45 @@ void gemm_nt_big_kernel(const BigLaunch L) {
     const bool tail_dead = (KT - 1) * kBK + ld_kc >= K;
     const float alpha = descale_factor(P.scale_a, P.scale_b, P.ex.scale_inv);
 
-    {
-        constexpr int LA = MI * 2 * 16 / 8 / kBigWaves;  // wave-level loads of the A tile per wave per stage
-        constexpr int LB = kBigLB;
-        constexpr int NL = LA + LB;                      // loads per wave per K-tile
-        static_assert(NL % 4 == 0, "the loads are queued in four equal portions");
-        const int wm = (wave >> 1) * (MI * 16), wn = (wave & 1) * 128;
+    constexpr int LA = MI * 2 * 16 / 8 / kBigWaves;  // wave-level loads of the A tile per wave per stage
+    constexpr int LB = kBigLB;
+    constexpr int NL = LA + LB;                      // loads per wave per K-tile
+    static_assert(NL % 4 == 0, "the loads are queued in four equal portions");
+    const int wm = (wave >> 1) * (MI * 16), wn = (wave & 1) * 128;
 
+    v4f acc[MI][kBigNJ];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < kBigNJ; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    // The K loop.  kAT: the A operand is given as its transpose, a [K, M] tensor (what wgrad has of dY: its reduction
+    // index, the token, is the row index).  Its K-tiles lie in LDS as they lie in memory, 128 rows of k with 256 (whole
+    // tiles) or 128 (half tiles) bytes of m each, and the 16 x 128 fragments are gathered with the transposing LDS read,
+    // exactly as for a transposed B operand.  Operand layout is a property of the problem, decided per workgroup: a
+    // launch mixes dgrad (A plain) and wgrad (A transposed) tiles.
+    auto kloop = [&](auto at_tag) {
+        constexpr bool kAT = decltype(at_tag)::value;
         uint32_t a_off[LA], b_off[LB];
 #pragma unroll
-        for (int i = 0; i < LA; ++i)   // rows >= M fall past the descriptor: zeros
-            a_off[i] = (uint32_t)(m0 + (wave + kBigWaves * i) * 8 + (lane >> 3)) * (uint32_t)K + ld_kc;
+        for (int i = 0; i < LA; ++i) {
+            if constexpr (kAT && MI == 8) {
+                // as the transposed B below: 4 rows of k per wave-level load, 16 chunks of m each
+                const int k = (wave + kBigWaves * i) * 4 + (lane >> 4);
+                const int chunk = (lane & 15) ^ ((k & 7) | (((k >> 5) & 1) << 3));
+                a_off[i] = (uint32_t)k * (uint32_t)M + (uint32_t)(m0 + chunk * 16);
+            } else if constexpr (kAT) {
+                // half tiles: 128 bytes of m per row of k, 8 rows of k per wave-level load; chunk c of row k is stored
+                // at chunk c ^ ((k / 2 mod 4) | 4 (k / 32 mod 2)): the 8 rows one transposing read touches, and the
+                // two 16-lane groups that go through LDS together, then use 16 different 16-byte bank groups
+                const int k = (wave + kBigWaves * i) * 8 + (lane >> 3);
+                const int chunk = (lane & 7) ^ (((k >> 1) & 3) | (((k >> 5) & 1) << 2));
+                a_off[i] = (uint32_t)k * (uint32_t)M + (uint32_t)(m0 + chunk * 16);
+            } else {
+                // rows >= M fall past the descriptor: zeros
+                a_off[i] = (uint32_t)(m0 + (wave + kBigWaves * i) * 8 + (lane >> 3)) * (uint32_t)K + ld_kc;
+            }
+        }
 #pragma unroll
         for (int i = 0; i < LB; ++i) {
             if constexpr (kBT) {
@@ -348,13 +377,7 @@ void gemm_nt_big_kernel(const BigLaunch L) {
             }
         }
         // byte distance between K-tiles in memory
-        const int a_step = kBK, b_step = kBT ? kBK * N : kBK;
-
-        v4f acc[MI][kBigNJ];
-#pragma unroll
-        for (int i = 0; i < MI; ++i)
-#pragma unroll
-            for (int j = 0; j < kBigNJ; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+        const int a_step = kAT ? kBK * M : kBK, b_step = kBT ? kBK * N : kBK;
 
         // load number `l` (0 .. NL-1, A loads first) of K-tile `ktile` straight into its LDS stage, ktile mod NS
         auto issue = [&](int ktile, int l) {
@@ -368,8 +391,10 @@ void gemm_nt_big_kernel(const BigLaunch L) {
         // lanes whose chunk lies at k >= K get an offset past the descriptor and so read zeros.
         auto poison_tail = [&]() {
             if (tail_dead) {
+                if constexpr (!kAT) {   // (rows k >= K of a transposed operand fall past its descriptor by themselves)
 #pragma unroll
-                for (int i = 0; i < LA; ++i) a_off[i] = 0xfffffff0u;
+                    for (int i = 0; i < LA; ++i) a_off[i] = 0xfffffff0u;
+                }
                 if constexpr (!kBT) {
 #pragma unroll
                     for (int i = 0; i < LB; ++i) b_off[i] = 0xfffffff0u;
@@ -383,15 +408,32 @@ void gemm_nt_big_kernel(const BigLaunch L) {
         const int fk = (lane >> 4) * 2;
         const int a_rd0 = lds_off16(wm + frow, fk), a_rd1 = lds_off16(wm + frow, fk + 1);
         const int b_rd0 = lds_off16(wn + frow, fk), b_rd1 = lds_off16(wn + frow, fk + 1);
-        // half h (0 / 1) of a fragment = one 128-bit LDS read
-        auto rd_a = [&](int s, int i, int h) -> v4i {
-            return *reinterpret_cast<const v4i*>(&sA[s][(h ? a_rd1 : a_rd0) + i * 2048]);
-        };
-        // transposed B: lane u of a 16-lane group (which serves k 32 (lane / 16) .. + 31) addresses row k0 + u / 2,
+        // transposed operands: lane u of a 16-lane group (which serves k 32 (lane / 16) .. + 31) addresses row k0 + u / 2,
         // half u % 2 of the block's 16-byte chunk; quarter t of the fragment is k0 = 32 (lane / 16) + 8 t
         const int bt_row = (lane & 15) >> 1;
         const int bt_base = ((lane >> 4) * 32 + bt_row) * 256 + ((((wave & 1) ^ ((lane >> 4) & 1))) << 7) + (lane & 1) * 8;
         const int bt_x = bt_row << 4;
+        // the same for A: the wave's blocks are chunks 8 (wave / 2) + i of a 256-byte row (whole tiles), chunks
+        // 4 (wave / 2) + i of a 128-byte row (half tiles, swizzle (k / 2 mod 4) | 4 (k / 32 mod 2))
+        const int at_base = MI == 8 ? ((lane >> 4) * 32 + bt_row) * 256 + ((((wave >> 1) ^ ((lane >> 4) & 1))) << 7) + (lane & 1) * 8
+                                    : ((lane >> 4) * 32 + bt_row) * 128 + ((((wave >> 1) ^ ((lane >> 4) & 1))) << 6) + (lane & 1) * 8;
+        const int at_x = MI == 8 ? bt_row << 4 : ((bt_row >> 1) & 3) << 4;
+        constexpr int at_pitch = MI == 8 ? 256 : 128;
+        // half h (0 / 1) of a fragment = one 128-bit LDS read, or two transposing 64-bit reads
+        auto rd_a = [&](int s, int i, int h) -> v4i {
+            if constexpr (kAT) {
+                typedef int v2i __attribute__((ext_vector_type(2)));
+                typedef __attribute__((address_space(3))) v2i* tr_ptr;
+                int x = at_x;
+                if constexpr (MI == 4) asm volatile("" : "+v"(x));
+                uint8_t* p = &sA[s][at_base + ((i << 4) ^ x) + h * (2 * 8 * at_pitch)];
+                const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((tr_ptr)p);
+                const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((tr_ptr)(p + 8 * at_pitch));
+                return (v4i){lo.x, lo.y, hi.x, hi.y};
+            } else {
+                return *reinterpret_cast<const v4i*>(&sA[s][(h ? a_rd1 : a_rd0) + i * 2048]);
+            }
+        };
         auto rd_b = [&](int s, int j, int h) -> v4i {
             if constexpr (kBT) {
                 typedef int v2i __attribute__((ext_vector_type(2)));
@@ -629,7 +671,15 @@ void gemm_nt_big_kernel(const BigLaunch L) {
         front(No{}, NoBarrier{}, f);
         back(No{}, No{}, f);
         }
+    };
+    if constexpr (kBT) {
+        if (P.at) kloop(std::true_type{});   // uniform for the workgroup
+        else kloop(std::false_type{});
+    } else {
+        kloop(std::false_type{});
+    }
 
+    {
         // output type, accumulation and bias are properties of the problem, not of the kernel (fp8 outputs apart)
         auto epilogue = [&](auto bias_tag, const float (*bv)[4]) {
             constexpr bool kBias = decltype(bias_tag)::value;

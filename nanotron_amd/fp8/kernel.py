@@ -110,6 +110,17 @@ def b_transposed_supported(M: int, N: int, K: int) -> bool:
             and (M + 256) * K < 2 ** 31 and (N + 256) * K < 2 ** 31)
 
 
+# Module switch: False makes wgrad GEMMs take a materialised transpose of the output gradient (kernel.py:44).
+READ_A_TRANSPOSED = True
+
+
+def a_transposed_supported(M: int, N: int, K: int) -> bool:
+    """Whether the library reads BOTH operands of D[M,N] = A[M,K] . B[N,K]^T from their transposes, [K, M] and [K, N]
+    tensors (`ntfp8_gemm_desc.a_transposed` next to `b_transposed`): the wgrad form, dW = dY^T . X with dY[tokens, out]
+    and X[tokens, in] as they are."""
+    return READ_A_TRANSPOSED and M % 16 == 0 and b_transposed_supported(M, N, K)
+
+
 def needs_transposed_copy(rows: int, cols: int, other: int = 4096) -> bool:
     """Whether a [rows, cols] fp8 tensor that a backward GEMM reduces over its rows (the weight in dgrad, the input in
     wgrad; src/nanotron/fp8/linear.py:104-109) should be quantised together with its transposed copy: only if the
@@ -120,8 +131,9 @@ def needs_transposed_copy(rows: int, cols: int, other: int = 4096) -> bool:
 
 def _gemm_nt_batch(problems):
     """Several independent `_gemm_nt` problems, given as tuples (a, b, out_dtype, accumulate_into[, b_transposed[,
-    bias]]), in one call of the library: GEMMs with the same operand formats share launches.  With `b_transposed`
-    the tensor `b` is the [K, N] transpose of the operand.  Returns the outputs in order."""
+    bias[, a_transposed]]]), in one call of the library: GEMMs with the same operand formats share launches.  With
+    `b_transposed` the tensor `b` is the [K, N] transpose of the operand, with `a_transposed` the tensor `a` its [K, M]
+    transpose.  Returns the outputs in order."""
     descs = (nt.GemmDesc * len(problems))()
     outs, keep = [], []
     dev = problems[0][0].device
@@ -129,9 +141,11 @@ def _gemm_nt_batch(problems):
         a, b, out_dtype, accumulate_into = prob[:4]
         bt = bool(prob[4]) if len(prob) > 4 else False
         bias = prob[5] if len(prob) > 5 else None
-        assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0 if bt else 1], (tuple(a.shape), tuple(b.shape), bt)
+        at = bool(prob[6]) if len(prob) > 6 else False
+        assert a.dim() == 2 and b.dim() == 2 and a.shape[0 if at else 1] == b.shape[0 if bt else 1], \
+            (tuple(a.shape), tuple(b.shape), bt, at)
         assert a.device == dev and b.device == dev
-        M, K = a.shape
+        K, M = a.shape if at else (a.shape[1], a.shape[0])
         N = b.shape[1 if bt else 0]
         a, ma = _bytes_and_meta(a)
         b, mb = _bytes_and_meta(b)
@@ -148,6 +162,7 @@ def _gemm_nt_batch(problems):
         d.M, d.N, d.K = M, N, K
         d.fmt_a, d.fmt_b, d.d_dtype, d.accumulate = _FMT[ma.dtype], _FMT[mb.dtype], nt.TORCH_TO_NT[out.dtype], acc
         d.b_transposed = 1 if bt else 0
+        d.a_transposed = 1 if at else 0
         outs.append(out)
         keep.append((a, b, bias))
     nt.check(nt.lib.ntfp8_gemm_batch(descs, len(problems), nt.stream_ptr(dev)), "ntfp8_gemm_batch")
@@ -156,22 +171,31 @@ def _gemm_nt_batch(problems):
 
 def _operands(mat_a: FP8Tensor, transpose_a: bool, mat_b: FP8Tensor, transpose_b: bool,
               accumulate_into: Optional[torch.Tensor] = None, allow_bt: bool = True):
-    """(A, B, b_transposed) of the library's D = A . B^T for the reference's D = op_b(B) . op_a(A) (kernel.py:43-44).
+    """(A, B, b_transposed, a_transposed) of the library's D = A . B^T for the reference's D = op_b(B) . op_a(A)
+    (kernel.py:43-44).
 
     Where the reference transposes mat_a (tex.fp8_transpose, kernel.py:43) the library can read it as it is
     (`b_transposed`): that is taken when mat_a carries no transposed copy yet and the shape qualifies; otherwise the
-    copy is used (and made, once, if it does not exist)."""
+    copy is used (and made, once, if it does not exist).  The same for mat_b (kernel.py:44, `a_transposed`), which the
+    library serves next to an untransposed mat_a: the wgrad form."""
     assert mat_a.device != torch.device("cpu") and mat_b.device != torch.device("cpu"), \
         "The tensors must be on a CUDA device in order to use the FP8 kernel!!"
     assert hasattr(mat_a, "fp8_meta") and hasattr(mat_b, "fp8_meta"), "operands must be FP8Tensors"
-    b_ = mat_b.transposed() if transpose_b else mat_b   # the library's A: always K-contiguous
     if transpose_a:
-        return b_, mat_a, False
-    aligned = all(t is None or t.data_ptr() % 16 == 0 for t in (mat_a, b_, accumulate_into))   # 16-byte loads / stores
-    if allow_bt and getattr(mat_a, "_transposed", None) is None and mat_a.dim() == 2 and mat_a.is_contiguous() and aligned and \
-            b_transposed_supported(b_.shape[0], mat_a.shape[1], mat_a.shape[0]):
-        return b_, mat_a, True
-    return b_, mat_a.transposed(), False
+        return (mat_b.transposed() if transpose_b else mat_b), mat_a, False, False
+    aligned = all(t is None or t.data_ptr() % 16 == 0 for t in (mat_a, mat_b, accumulate_into))   # 16-byte loads / stores
+    plain_a = allow_bt and getattr(mat_a, "_transposed", None) is None and mat_a.dim() == 2 and mat_a.is_contiguous() and aligned
+    if transpose_b:
+        # D[cols of mat_b, cols of mat_a], reduction over the rows of both
+        if plain_a and getattr(mat_b, "_transposed", None) is None and mat_b.dim() == 2 and mat_b.is_contiguous() and \
+                a_transposed_supported(mat_b.shape[1], mat_a.shape[1], mat_a.shape[0]):
+            return mat_b, mat_a, True, True
+        b_ = mat_b.transposed()
+    else:
+        b_ = mat_b   # the library's A: K-contiguous
+    if plain_a and b_.data_ptr() % 16 == 0 and b_transposed_supported(b_.shape[0], mat_a.shape[1], mat_a.shape[0]):
+        return b_, mat_a, True, False
+    return b_, mat_a.transposed(), False, False
 
 
 @torch.no_grad()
@@ -182,8 +206,8 @@ def fp8_matmul_pair(first: dict, second: dict):
     probs = []
     for kw in (first, second):
         acc = kw.get("accumulate_into")
-        A, B, bt = _operands(kw["mat_a"], kw["transpose_a"], kw["mat_b"], kw["transpose_b"], acc)
-        probs.append((A, B, (kw.get("out_dtype") or torch.float32) if acc is None else torch.float32, acc, bt))
+        A, B, bt, at = _operands(kw["mat_a"], kw["transpose_a"], kw["mat_b"], kw["transpose_b"], acc)
+        probs.append((A, B, (kw.get("out_dtype") or torch.float32) if acc is None else torch.float32, acc, bt, None, at))
     return _gemm_nt_batch(probs)
 
 
@@ -224,7 +248,7 @@ def fp8_matmul_kernel(
         a_ = mat_a if transpose_a else mat_a.transposed()  # kernel.py:43
         b_ = mat_b.transposed() if transpose_b else mat_b  # kernel.py:44
         return _gemm_nt_fp8(b_, a_, out_dtype, out_state, out_with_transpose, bias)
-    A, B, bt = _operands(mat_a, transpose_a, mat_b, transpose_b, accumulate_into, allow_bt=bias is None)
+    A, B, bt, at = _operands(mat_a, transpose_a, mat_b, transpose_b, accumulate_into, allow_bt=bias is None)
     if bt:
-        return _gemm_nt_batch([(A, B, out_dtype or torch.float32, accumulate_into, True)])[0]
+        return _gemm_nt_batch([(A, B, out_dtype or torch.float32, accumulate_into, True, None, at)])[0]
     return _gemm_nt(A, B, out_dtype or torch.float32, accumulate_into, bias)

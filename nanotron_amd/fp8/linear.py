@@ -6,7 +6,7 @@ from torch import nn
 
 from nanotron_amd.fp8.constants import INITIAL_AMAX, INITIAL_SCALING_FACTOR
 from nanotron_amd.fp8.dtypes import DTypes
-from nanotron_amd.fp8.kernel import fp8_matmul_kernel, fp8_matmul_pair, needs_transposed_copy
+from nanotron_amd.fp8.kernel import a_transposed_supported, fp8_matmul_kernel, fp8_matmul_pair, needs_transposed_copy
 from nanotron_amd.fp8.meta import FP8Meta
 from nanotron_amd.fp8.parameter import FP8Parameter
 from nanotron_amd.fp8.tensor import DelayedScaling, FP8Tensor, cast_with_scale, update_scaling_factor
@@ -267,8 +267,13 @@ class _FP8Matmul(torch.autograd.Function):
 
         if type(grad_output) == torch.Tensor:
             g2d = grad_output.reshape(-1, grad_output.shape[-1]).contiguous()
+            # wgrad reduces over the rows of dY: it needs the transposed bytes (kernel.py:44) unless the library reads
+            # dY as it is, next to an input it also reads as it is
+            x_plain = getattr(input, "_transposed", None) is None
+            with_t = weight.requires_grad and not (
+                x_plain and a_transposed_supported(g2d.shape[1], input.shape[1], g2d.shape[0]))
             grad_output = FP8Tensor(g2d, dtype=DTypes.FP8E5M2, state=scaling["output_grad"] if scaling else None,
-                                    with_transpose=weight.requires_grad)
+                                    with_transpose=with_t)
 
         wants_dx = ctx.needs_input_grad[0] or (ctx.has_handle and ctx.needs_input_grad[6])
         grad_input = None

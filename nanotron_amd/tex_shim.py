@@ -116,13 +116,14 @@ def te_gemm(A: torch.Tensor, A_scale_inverse: torch.Tensor, A_type, transa: bool
     """cuBLASLt's column-major GEMM on row-major torch tensors, written into D:
         transa=True,  transb=False:  D[B.rows, A.rows] = B . A^T        (the form the reference issues)
         transa=False, transb=False:  D[B.rows, A.cols] = B . A          (A is read as it is, no transposed copy)
+        transa=False, transb=True:   D[B.cols, A.cols] = B^T . A        (both read as they are: the wgrad form)
     times A_scale_inverse * B_scale_inverse, fp32 accumulation, plus `bias` (one value per column of D) if it is
     not empty, one rounding to D's type; `accumulate` adds into an fp32 D.  With an fp8 `D_type`, D receives
-    sat_rne_fp8(result * D_scale) and D_amax max(D_amax, max|result|).  transb=True, `grad` (bias gradient) and a
-    non-empty `pre_gelu_out` are not served.  `workspace`, `use_split_accumulator` and `math_sm_count` have no
+    sat_rne_fp8(result * D_scale) and D_amax max(D_amax, max|result|).  transa=True with transb=True, `grad` (bias
+    gradient) and a non-empty `pre_gelu_out` are not served.  `workspace`, `use_split_accumulator` and `math_sm_count` have no
     meaning here: the kernels need no workspace and the matrix cores always accumulate in fp32."""
-    if transb:
-        raise RuntimeError("te_gemm: transb=True is not supported (pass the operand K-contiguous, as the reference does)")
+    if transb and transa:
+        raise RuntimeError("te_gemm: transa=True with transb=True is not supported")
     if grad and bias is not None and bias.numel() > 0:
         raise RuntimeError("te_gemm: the bias-gradient epilogue (grad=True with a bias) is not supported")
     if pre_gelu_out is not None and pre_gelu_out.numel() > 0:
@@ -132,7 +133,7 @@ def te_gemm(A: torch.Tensor, A_scale_inverse: torch.Tensor, A_type, transa: bool
     a = A.detach().as_subclass(torch.Tensor).contiguous()
     b = B.detach().as_subclass(torch.Tensor).contiguous()
     dev = a.device
-    M, K = b.shape                      # rows of D, reduction length
+    M, K = (b.shape[1], b.shape[0]) if transb else b.shape   # rows of D, reduction length
     if transa:
         N, Ka = a.shape
     else:
@@ -149,6 +150,7 @@ def te_gemm(A: torch.Tensor, A_scale_inverse: torch.Tensor, A_type, transa: bool
     p.A, p.scale_a, p.fmt_a = b.data_ptr(), sb.data_ptr(), _fmt(B_type)
     p.B, p.scale_b, p.fmt_b = a.data_ptr(), sa.data_ptr(), _fmt(A_type)
     p.b_transposed = 0 if transa else 1
+    p.a_transposed = 1 if transb else 0
     p.scales_are_inverse = 1
     p.D, p.M, p.N, p.K = D.data_ptr(), M, N, K
     p.accumulate = 1 if accumulate else 0

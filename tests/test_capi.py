@@ -173,13 +173,16 @@ def test_fp8_output_and_transposed_operand_requests_are_validated_before_any_lau
     assert L.ntfp8_amax_finalize(P, 0, 0, P + 4096, None, 4, P + 256, None, None) == -3           # length without a history
     assert L.ntfp8_amax_finalize(P, 0, 500, P + 4096, None, 0, P + 256, None, None) == -3
     assert L.ntfp8_amax_finalize(P, 0, 0, P + 4098, None, 0, P + 256, None, None) == -4
-    assert ctypes.sizeof(nt.GemmDesc) == 128
+    assert ctypes.sizeof(nt.GemmDesc) == 136
     # bias: dtype, alignment, overlap with the output, not together with a transposed B operand
     B0 = P + (5 << 20)
     assert L.ntfp8_gemm_batch(desc(bias=B0, bias_dtype=7), 1, None) == -2
     assert L.ntfp8_gemm_batch(desc(bias=B0 + 2, bias_dtype=0), 1, None) == -4
     assert L.ntfp8_gemm_batch(desc(bias=P + (3 << 20) + 128, bias_dtype=2), 1, None) == -7
     assert L.ntfp8_gemm_batch(desc(bias=B0, bias_dtype=2, b_transposed=1), 1, None) == -5
+    # a transposed A operand: only next to a transposed B, M a multiple of 16
+    assert L.ntfp8_gemm_batch(desc(a_transposed=1), 1, None) == -5
+    assert L.ntfp8_gemm_batch(desc(M=250, a_transposed=1, b_transposed=1), 1, None) == -5
 
 
 def test_a_failed_batch_has_launched_nothing():

@@ -209,3 +209,128 @@ def test_operator_falls_back_to_a_transposed_copy_when_the_direct_read_does_not_
     W3 = from_bytes(O.cast_to_fp8(w3, one, O.E4M3), 1.0, O.E4M3)
     assert _operands(W3, False, X, False)[2] is False
     assert torch.equal(fp8_matmul_kernel(W3, False, X, False, False).cpu(), x @ w3)
+
+
+# ------------------------------------------------------------------------------------------ both operands transposed
+def test_a_and_b_transposed_integer_sweep_singly_and_batched():
+    """The wgrad form: D[M,N] = A^T . B with A given as [K, M] and B as [K, N] (`a_transposed` next to `b_transposed`).
+    Integer operands: exact in any order, so whole tiles, half tiles, ragged edges, K tails, every format pair and
+    output type must equal the fp64 product; then all of them in one call next to plain and B-transposed problems."""
+    from nanotron_amd.fp8.kernel import _gemm_nt_batch
+
+    rng = torch.Generator().manual_seed(271828)
+    one = torch.tensor(1.0)
+    shapes = [(2304, 2048, 400), (4096, 4352, 256), (144, 144, 256), (1008, 272, 1040), (6144, 4096, 512)]
+    for _ in range(9):
+        shapes.append((16 * int(torch.randint(9, 88, (1,), generator=rng)), 16 * int(torch.randint(9, 88, (1,), generator=rng)),
+                       16 * int(torch.randint(16, 130, (1,), generator=rng))))
+    problems, wants = [], []
+    for case, (M, N, K) in enumerate(shapes):
+        fa, fb = [(O.E5M2, O.E4M3), (O.E4M3, O.E4M3), (O.E4M3, O.E5M2), (O.E5M2, O.E5M2)][case % 4]
+        at = torch.randint(-4, 5, (K, M), generator=rng).float()
+        bt = torch.randint(-4, 5, (K, N), generator=rng).float()
+        At = from_bytes(O.cast_to_fp8(at, one, fa), 0.5, fa)
+        Bt = from_bytes(O.cast_to_fp8(bt, one, fb), 2.0, fb)
+        want = (at.double().t() @ bt.double()).float()
+        od = (torch.float32, torch.bfloat16, torch.float16)[case % 3]
+        got = _gemm_nt_batch([(At, Bt, od, None, True, None, True)])[0]
+        assert got.shape == (M, N) and got.dtype == od
+        assert torch.equal(got.cpu(), want.to(od)), (M, N, K, fa, fb, od)
+        if case % 3 == 0:
+            acc = torch.randint(-50, 50, (M, N), generator=rng).float()
+            accg = acc.cuda()
+            out = _gemm_nt_batch([(At, Bt, torch.float32, accg, True, None, True)])[0]
+            assert out.data_ptr() == accg.data_ptr() and torch.equal(out.cpu(), want + acc)
+        problems.append((At, Bt, od, None, True, None, True))
+        wants.append(want.to(od))
+    # a dgrad-shaped problem (A plain, B transposed) and a plain one ride along: operand layout is per problem
+    a = torch.randint(-4, 5, (640, 512), generator=rng).float()
+    b_t = torch.randint(-4, 5, (512, 272), generator=rng).float()
+    b = torch.randint(-4, 5, (272, 512), generator=rng).float()
+    A = from_bytes(O.cast_to_fp8(a, one, O.E5M2), 1.0, O.E5M2)
+    problems.append((A, from_bytes(O.cast_to_fp8(b_t, one, O.E4M3), 1.0, O.E4M3), torch.float32, None, True))
+    wants.append(a @ b_t)
+    problems.append((A, from_bytes(O.cast_to_fp8(b, one, O.E4M3), 1.0, O.E4M3), torch.float32, None))
+    wants.append(a @ b.t())
+    for got, want in zip(_gemm_nt_batch(problems), wants):
+        assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("mnk", [(768, 512, 384), (4096, 4096, 2048), (1536, 1024, 4096), (6144, 4096, 4096)])
+def test_a_transposed_random_operands_equal_the_gemm_on_materialised_transposes(mnk):
+    """Same tiles, same MFMA order: reading dY and X as they are must give the bits of the GEMM on their transposed
+    copies, whole tiles and half-tile tail alike; and the oracle's result within the GEMM tolerance."""
+    from nanotron_amd.fp8 import FP8Tensor
+    from nanotron_amd.fp8.kernel import _gemm_nt, _gemm_nt_batch
+
+    M, N, K = mnk
+    At = FP8Tensor(O.normal_tensor(M, (K, M), 1e-2, torch.bfloat16).cuda(), _dt(O.E5M2), with_transpose=True)
+    Bt = FP8Tensor(O.normal_tensor(N + 1, (K, N), 1.0, torch.bfloat16).cuda(), _dt(O.E4M3), with_transpose=True)
+    for od in (torch.float32, torch.bfloat16):
+        got = _gemm_nt_batch([(At, Bt, od, None, True, None, True)])[0]
+        ref = _gemm_nt(At.transposed(), Bt.transposed(), od, None)
+        assert torch.equal(got, ref)
+    r = O.gemm_nt(At.transposed().cpu().as_subclass(torch.Tensor), O.E5M2, At.fp8_meta.scale.cpu(),
+                  Bt.transposed().cpu().as_subclass(torch.Tensor), O.E4M3, Bt.fp8_meta.scale.cpu())
+    assert O.rel_l2(_gemm_nt_batch([(At, Bt, torch.float32, None, True, None, True)])[0].cpu(), r) <= 1e-3
+
+
+def test_a_transposed_requests_the_kernels_do_not_serve_are_refused():
+    from nanotron_amd import _native as nt
+    from nanotron_amd.fp8 import FP8Tensor
+    from nanotron_amd.fp8.kernel import a_transposed_supported
+
+    dev = torch.device("cuda", 0)
+
+    def call(M, N, K, bt=1):
+        a = FP8Tensor(torch.randn(K, M, device=dev), _dt(O.E4M3))
+        b = FP8Tensor(torch.randn(K, N, device=dev), _dt(O.E4M3))
+        out = torch.empty(M, N, dtype=torch.float32, device=dev)
+        d = nt.GemmDesc()
+        d.A, d.scale_a, d.B, d.scale_b, d.D = a.data_ptr(), a.fp8_meta.scale.data_ptr(), b.data_ptr(), b.fp8_meta.scale.data_ptr(), out.data_ptr()
+        d.M, d.N, d.K, d.fmt_a, d.fmt_b, d.d_dtype, d.b_transposed, d.a_transposed = M, N, K, nt.E4M3, nt.E4M3, nt.F32, bt, 1
+        rc = nt.lib.ntfp8_gemm_batch((nt.GemmDesc * 1)(d), 1, nt.stream_ptr(dev))
+        torch.cuda.synchronize()
+        return rc
+
+    assert a_transposed_supported(256, 256, 256) and call(256, 256, 256) == 0
+    assert call(256, 256, 256, bt=0) == -5                       # only next to a transposed B
+    for M, N, K in [(250, 256, 256), (256, 250, 256), (128, 256, 256), (256, 256, 128)]:
+        assert not a_transposed_supported(M, N, K)
+        assert call(M, N, K) == -5, (M, N, K)
+
+
+def test_linear_backward_reads_the_output_gradient_as_it_is():
+    """FP8Linear's wgrad takes dY without a transposed copy when the shape allows it, and gives the bits of the path on
+    transposed copies."""
+    import nanotron_amd.fp8.kernel as K
+    from nanotron_amd.fp8 import DTypes, FP8Linear, FP8Parameter, FP8Tensor
+
+    T, H, I = 384, 512, 768
+    w = O.normal_tensor(1, (I, H), 0.05, torch.bfloat16)
+    seen, results = [], []
+    orig = FP8Tensor.__new__
+
+    def spy(cls, tensor, dtype, **kw):
+        if dtype == DTypes.FP8E5M2:
+            seen.append(bool(kw.get("with_transpose")))
+        return orig(cls, tensor, dtype, **kw)
+
+    for direct in (True, False):
+        K.READ_A_TRANSPOSED = direct
+        FP8Tensor.__new__ = spy
+        try:
+            lin = FP8Linear(H, I, bias=False, device="cuda", dtype=torch.bfloat16, out_dtype=torch.bfloat16, delayed_scaling=True)
+            lin.weight = FP8Parameter(w.cuda(), DTypes.FP8E4M3)
+            outs = []
+            for step in range(3):
+                x = O.normal_tensor(10 + step, (T, H), 1.0, torch.bfloat16).cuda().requires_grad_(True)
+                lin(x).backward(O.normal_tensor(20 + step, (T, I), 1e-2, torch.bfloat16).cuda())
+                outs += [x.grad.clone(), lin.weight.main_grad.clone()]
+            results.append(outs)
+        finally:
+            K.READ_A_TRANSPOSED = True
+            FP8Tensor.__new__ = orig
+    assert seen == [False] * 3 + [True] * 3
+    for a, b in zip(*results):
+        assert torch.equal(_bits(a), _bits(b))

@@ -188,6 +188,12 @@ def test_te_gemm_integer_operands_bit_exact_all_arguments():
             tex.te_gemm(at, sa_inv, tex.DType.kFloat8E4M3, False, bq, sb_inv, tex.DType.kFloat8E5M2, False,
                         D, e, tex.DType.kFloat32, e, torch.tensor([]), tex.DType.kFloat32, e, False, ws, 16, False, True, 0)
             assert torch.equal(D.cpu(), want)
+            if M % 16 == 0:
+                bt = O.cast_to_fp8(b.t().contiguous(), one, O.E5M2).cuda()   # B as [K, M] too: the wgrad form, transb=True
+                D = torch.empty(M, N, device="cuda")
+                tex.te_gemm(at, sa_inv, tex.DType.kFloat8E4M3, False, bt, sb_inv, tex.DType.kFloat8E5M2, True,
+                            D, e, tex.DType.kFloat32, e, torch.tensor([]), tex.DType.kFloat32, e, False, ws, 16, False, True, 0)
+                assert torch.equal(D.cpu(), want)
     with pytest.raises(RuntimeError):
         tex.te_gemm(aq, sa_inv, tex.DType.kFloat8E4M3, True, bq, sb_inv, tex.DType.kFloat8E5M2, True,
                     D, e, tex.DType.kFloat32, e, torch.tensor([]), tex.DType.kFloat32, e, False, ws, 16, False, True, 0)
