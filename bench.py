@@ -54,7 +54,9 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=20)
     p.add_argument("--warmup", type=int, default=5)
-    p.add_argument("--workload", choices=["linear", "quant", "probe"], default="linear")
+    p.add_argument("--workload", choices=["linear", "quant", "probe", "vendor-gemm"], default="linear",
+                   help="linear: the headline step; quant: configuration 2; probe: a few launches for counter runs; "
+                        "vendor-gemm: hipBLASLt's fp8 GEMM next to this library's on the forward shapes")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--weight-stream", action="store_true",
                    help="re-quantise the weights on a second stream (measured: no gain, the GEMMs are power-bound)")
@@ -66,6 +68,8 @@ def parse():
                         "reference's way, kernel.py:44) instead of letting the GEMM read dY as it is")
     p.add_argument("--kernel-reps", type=int, default=0,
                    help="also time each GEMM shape in isolation with this many back-to-back launches (0 = skip)")
+    p.add_argument("--operand-sets", type=int, default=4,
+                   help="vendor-gemm: operand sets walked round robin (1 = operands stay in the memory-side cache)")
     p.add_argument("--fp8-activations", action="store_true",
                    help="every linear returns its output as an e4m3 FP8Tensor quantised in the GEMM epilogue "
                         "(no bf16 activation is written); not the headline configuration")
@@ -494,13 +498,14 @@ def cpu_baseline_quant():
 
 # ------------------------------------------------------------------------------------ counter probe
 def probe(device):
-    """A handful of launches for `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs: one plain copy of
-    known size (the calibration for the counters), the fused quantise kernel on the benchmark tensor,
-    and one GEMM of every kind on the O-projection and gate shapes.  Prints what was launched."""
+    """A handful of launches for `rocprofv3 --pmc` runs, in this order: one plain copy of known size (the
+    calibration for FETCH_SIZE / WRITE_SIZE), the fused quantise kernels on the benchmark tensor (single format,
+    both formats), and for the O-projection and gate shapes the three GEMMs as FP8Linear issues them: forward, then
+    dgrad + wgrad in one batched call with W, X and dY read untransposed.  Prints what was launched."""
     import torch
 
     from nanotron_amd.fp8 import DTypes, FP8Tensor
-    from nanotron_amd.fp8.kernel import _gemm_nt
+    from nanotron_amd.fp8.kernel import _gemm_nt, _gemm_nt_batch
 
     src = torch.empty(128 * 1024 * 1024, dtype=torch.uint8, device=device).fill_(1)
     dst = torch.empty_like(src)
@@ -509,25 +514,86 @@ def probe(device):
     bufs, states = build_quant(device, nbuf=2)
     for i in range(3):
         quant_step(bufs, states, i)
+    quant_dual_kernel_ms(bufs, states, 2)
     g = torch.Generator(device="cpu").manual_seed(7)
     launched = {"copy": {"read_bytes": src.numel(), "write_bytes": src.numel()},
-                "quant_flat_kernel": {"elements": 4096 * 4096, "algorithmic_bytes": 3 * 4096 * 4096}}
+                "quant_flat_kernel": {"elements": 4096 * 4096, "algorithmic_bytes": 3 * 4096 * 4096},
+                "quant_flat_dual_kernel": {"elements": 4096 * 4096, "algorithmic_bytes": 4 * 4096 * 4096}}
     for name, K, N in (("o", 4096, 4096), ("gate", 4096, 14336)):
         x = torch.randn(TOKENS, K, generator=g).to(torch.bfloat16).to(device)
         w = (torch.randn(N, K, generator=g) * 0.02).to(device)
         gy = (torch.randn(TOKENS, N, generator=g) * 1e-3).to(torch.bfloat16).to(device)
-        xq = FP8Tensor(x, DTypes.FP8E4M3, with_transpose=True)
-        wq = FP8Tensor(w, DTypes.FP8E4M3, with_transpose=True)
-        gq = FP8Tensor(gy, DTypes.FP8E5M2, with_transpose=True)
+        xq, wq, gq = FP8Tensor(x, DTypes.FP8E4M3), FP8Tensor(w, DTypes.FP8E4M3), FP8Tensor(gy, DTypes.FP8E5M2)
         _gemm_nt(xq, wq, torch.bfloat16, None)
-        _gemm_nt(gq, wq.transposed(), torch.bfloat16, None)
-        _gemm_nt(gq.transposed(), xq.transposed(), torch.float32, None)
+        _gemm_nt_batch([(gq, wq, torch.bfloat16, None, True), (gq, xq, torch.float32, None, True, None, True)])
         launched[f"gemm_{name}"] = {"M": TOKENS, "N": N, "K": K,
                                     "algorithmic_bytes_fwd": TOKENS * K + N * K + 2 * TOKENS * N,
                                     "algorithmic_bytes_dgrad": TOKENS * N + N * K + 2 * TOKENS * K,
                                     "algorithmic_bytes_wgrad": TOKENS * N + TOKENS * K + 4 * N * K}
     torch.cuda.synchronize()
     print(json.dumps({"probe": launched}))
+
+
+# ------------------------------------------------------------------------------------ vendor library, for comparison
+def hipblaslt_reference(device, reps=30, nsets=4):
+    """The vendor's fp8 GEMM (hipBLASLt behind torch._scaled_mm, e4m3 x e4m3, bf16 output) on the forward shapes of
+    the workload, rotating operands as the step does.  A yardstick for the hand-written kernel, not part of the
+    product: nothing in nanotron_amd calls it."""
+    import torch
+
+    g = torch.Generator(device=device).manual_seed(3)
+    one = torch.tensor(1.0, device=device)
+    out = []
+    for name, K, N in LINEARS:
+        ops = []
+        for _ in range(nsets):
+            a = (torch.randn(TOKENS, K, generator=g, device=device) * 64).clamp(-448, 448).to(torch.float8_e4m3fn)
+            b = (torch.randn(N, K, generator=g, device=device) * 64).clamp(-448, 448).to(torch.float8_e4m3fn)
+            ops.append((a, b))
+        k = [0]
+
+        def fn():
+            a, b = ops[k[0] % len(ops)]
+            k[0] += 1
+            return torch._scaled_mm(a, b.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+
+        ms = event_time_ms(fn, reps, warm=6)
+        out.append({"gemm": f"{name}.fwd", "mnk": [TOKENS, N, K], "ms": round(ms, 4),
+                    "tflops": round(2.0 * TOKENS * N * K / ms / 1e9, 1)})
+        del ops
+    return out
+
+
+def own_forward_reference(device, reps=30, nsets=4):
+    """The same shapes, same rotation, through this library's forward GEMM (C ABI, outputs allocated beforehand, as
+    torch does for the vendor call from its caching allocator)."""
+    import torch
+
+    from nanotron_amd import _native as nt
+    from nanotron_amd.fp8 import DTypes, FP8Tensor
+
+    g = torch.Generator(device=device).manual_seed(3)
+    st = nt.stream_ptr(device)
+    out = []
+    for name, K, N in LINEARS:
+        ops = []
+        for _ in range(nsets):
+            a = FP8Tensor(torch.randn(TOKENS, K, generator=g, device=device).to(torch.bfloat16), DTypes.FP8E4M3)
+            b = FP8Tensor(torch.randn(N, K, generator=g, device=device).to(torch.bfloat16), DTypes.FP8E4M3)
+            ops.append((a, b, torch.empty(TOKENS, N, dtype=torch.bfloat16, device=device)))
+        k = [0]
+
+        def fn():
+            a, b, d = ops[k[0] % len(ops)]
+            k[0] += 1
+            nt.check(nt.lib.ntfp8_gemm(a.data_ptr(), nt.E4M3, a.fp8_meta.scale.data_ptr(), b.data_ptr(), nt.E4M3,
+                                       b.fp8_meta.scale.data_ptr(), d.data_ptr(), nt.BF16, TOKENS, N, K, 0, st), "ntfp8_gemm")
+
+        ms = event_time_ms(fn, reps, warm=6)
+        out.append({"gemm": f"{name}.fwd", "mnk": [TOKENS, N, K], "ms": round(ms, 4),
+                    "tflops": round(2.0 * TOKENS * N * K / ms / 1e9, 1)})
+        del ops
+    return out
 
 
 # ------------------------------------------------------------------------------------ main
@@ -555,6 +621,12 @@ def main():
 
     if args.workload == "probe":
         probe(device)
+        return
+    if args.workload == "vendor-gemm":
+        n = args.operand_sets
+        print(json.dumps({"workload": f"forward GEMMs of the step, e4m3 x e4m3 -> bf16, {n} rotating operand set(s)",
+                          "hipblaslt_scaled_mm": hipblaslt_reference(device, nsets=n),
+                          "ntfp8": own_forward_reference(device, nsets=n)}))
         return
     traffic = read_traffic(args)
     verified = None

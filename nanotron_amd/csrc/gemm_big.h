@@ -54,6 +54,13 @@ __device__ __forceinline__ v4i reg_load16(__amdgpu_buffer_rsrc_t r, uint32_t vof
     return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
 }
 __device__ __forceinline__ void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
+// 16 bytes of output to global memory, written through to memory as they are issued (sc0 sc1) and marked streaming
+// (nt).  An ordinary store leaves its line dirty in the XCD's L2; a tile's worth of output per CU then fills that L2,
+// and the lines are written back in one burst when the kernel ends.  Written through, the output drains while the
+// other waves still compute: 2.5 us less per round of tiles (4096^3: 58.0 -> 55.5 us; `nt` alone changes nothing).
+__device__ __forceinline__ void store16_through(void* p, v4i v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" ::"v"(p), "v"(v) : "memory");
+}
 
 // Epilogue of one wave: MI x NJ accumulator blocks of 16 x 16, block (i, j) at rows m_base + 16 i,
 // columns n_base + 16 j.  Descale, optional fp32 accumulate, one rounding, store.
@@ -89,7 +96,7 @@ __device__ __forceinline__ void store_wave_tile16(const v4f (&acc)[MI][NJ], void
                     // lane row q now holds n 8 (q / 2) .. + 7 of block j + (q & 1): x = first four, y = last four
                     const int n = n_base + (j + (q & 1)) * 16 + (q >> 1) * 8;
                     if (m < M && n < N)
-                        *reinterpret_cast<v4i*>(D + (int64_t)m * N + n) = (v4i){(int)x0, (int)x1, (int)y0, (int)y1};
+                        store16_through(D + (int64_t)m * N + n, (v4i){(int)x0, (int)x1, (int)y0, (int)y1});
                 }
             }
             return;
@@ -124,6 +131,7 @@ __device__ __forceinline__ void store_wave_tile16(const v4f (&acc)[MI][NJ], void
                 if constexpr (DT == NTFP8_F32) {
                     v4f o = {v[0], v[1], v[2], v[3]};
                     if constexpr (kAcc) o = o + old[j];
+                    // (fp32 outputs keep the ordinary store: written through they measured the same or slower)
                     *reinterpret_cast<v4f*>(dp) = o;
                 } else {
                     *reinterpret_cast<uint2*>(dp) = make_uint2(OutT<DT>::pack2(v[0], v[1]), OutT<DT>::pack2(v[2], v[3]));
@@ -146,13 +154,15 @@ __device__ __forceinline__ void store_wave_tile16(const v4f (&acc)[MI][NJ], void
     }
 }
 
-// 16 / 4 bytes per lane to global memory through a buffer descriptor; offsets past its size are dropped
+// 16 / 4 bytes per lane to global memory through a buffer descriptor; offsets past its size are dropped.  Cache policy
+// of the builtin's last argument on gfx950: bit 0 = sc0, bit 1 = nt, bit 4 = sc1 (written through, as store16_through).
+constexpr int kStoreThrough = 1 | 2 | 16;
 __device__ __forceinline__ void reg_store16(__amdgpu_buffer_rsrc_t r, uint32_t voff, v4i data) {
     typedef unsigned v4u __attribute__((ext_vector_type(4)));
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, data), r, voff, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, data), r, voff, 0, kStoreThrough);
 }
 __device__ __forceinline__ void reg_store4(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t data) {
-    __builtin_amdgcn_raw_buffer_store_b32(data, r, voff, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b32(data, r, voff, 0, kStoreThrough);
 }
 
 // fp8 epilogue of one wave (layout as store_wave_tile16); returns the lane's max|r| as a bit pattern.
