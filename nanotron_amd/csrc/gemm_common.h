@@ -14,7 +14,11 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
 constexpr int kBK = 128;     // bytes of K per LDS stage
-constexpr int kGroupM = 8;   // tile-order grouping for L2 reuse
+// Tile order: groups of kGroupM row-tiles, swept along N.  With 32 consecutive tiles of a round on one XCD (one per
+// CU), an XCD then works on a block of 4 row-tiles x 8 column-tiles: 4 A panels and 8 B panels per K step in its L2.
+// The transposed block (8 x 4, kGroupM = 8) moves the same number of panels and measured 2-6 % slower on the
+// one-round shapes (4096^3: 56.2 -> 52.8 us), 2 x 16 and 16 x 2 slower still on the long and wide ones.
+constexpr int kGroupM = 4;
 constexpr int kXcds = 8;     // workgroups are dealt round-robin to the 8 XCDs, each with its own L2
 
 // 16-byte chunk `kc` (0..7) of tile row `row`, swizzled so that the 16 lanes of a 128-bit LDS access
