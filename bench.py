@@ -659,6 +659,7 @@ def main():
     t0 = time.perf_counter()
     for i in range(args.steps):
         step(first + args.warmup + i)
+    host_ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3   # time the host needs to queue a step
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
@@ -666,6 +667,7 @@ def main():
     out = {
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "data": "synthetic",
+        "host_ms_per_step": round(host_ms_per_step, 4),
     }
     if args.workload == "linear":
         value = flops_step / (ms_per_step * 1e-3) / 1e12
