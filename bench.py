@@ -54,7 +54,7 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=20)
     p.add_argument("--warmup", type=int, default=5)
-    p.add_argument("--workload", choices=["linear", "quant", "probe", "vendor-gemm"], default="linear",
+    p.add_argument("--workload", choices=["linear", "quant", "probe", "vendor-gemm", "wg-timeline"], default="linear",
                    help="linear: the headline step; quant: configuration 2; probe: a few launches for counter runs; "
                         "vendor-gemm: hipBLASLt's fp8 GEMM next to this library's on the forward shapes")
     p.add_argument("--no-cpu-baseline", action="store_true")
@@ -535,6 +535,123 @@ def probe(device):
 
 
 # ------------------------------------------------------------------------------------ vendor library, for comparison
+def workgroup_timeline(device):
+    """Where a workgroup of the GEMM kernel spends its time, read from the kernel itself: the profiling build of the
+    library (libntfp8_stamps.so, -DNTFP8_STAMPS) stamps the 100 MHz wall clock five times per workgroup and records
+    the CU it ran on.  Four launches without a half-tile tail: one round at K = 4096 and at K = 14336, three rounds, and
+    the seven-round dgrad + wgrad launch of the down projection."""
+    import ctypes
+
+    import numpy as np
+    import torch
+
+    from nanotron_amd import _native as nt
+    from nanotron_amd.fp8 import DTypes, FP8Tensor
+
+    path = os.path.join(ROOT, "nanotron_amd", "libntfp8_stamps.so")
+    if not os.path.exists(path):
+        raise FileNotFoundError(f"{path}: build it with `python -m nanotron_amd.build`")
+    lib = ctypes.CDLL(path)
+    lib.ntfp8_gemm_batch.restype = ctypes.c_int
+    lib.ntfp8_gemm_batch.argtypes = [ctypes.POINTER(nt.GemmDesc), ctypes.c_int, ctypes.c_void_p]
+    lib.ntfp8_debug_stamps.restype = ctypes.c_int
+    lib.ntfp8_debug_stamps.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+    g = torch.Generator(device=device).manual_seed(1)
+
+    def q(shape, std, dt):
+        return FP8Tensor((torch.randn(shape, generator=g, device=device) * std).to(torch.bfloat16), dt)
+
+    st = nt.stream_ptr(device)
+
+    def run(probs):
+        d = (nt.GemmDesc * len(probs))()
+        for e, (a, b, out, bt, at, dd) in zip(d, probs):
+            e.A, e.scale_a, e.B, e.scale_b, e.D = (a.data_ptr(), a.fp8_meta.scale.data_ptr(), b.data_ptr(),
+                                                   b.fp8_meta.scale.data_ptr(), out.data_ptr())
+            (e.K, e.M) = a.shape if at else a.shape[::-1]
+            e.N = b.shape[1] if bt else b.shape[0]
+            e.fmt_a = 0 if a.fp8_meta.dtype == DTypes.FP8E4M3 else 1
+            e.fmt_b = 0 if b.fp8_meta.dtype == DTypes.FP8E4M3 else 1
+            e.d_dtype, e.accumulate, e.b_transposed, e.a_transposed = dd, 0, int(bt), int(at)
+        rc = lib.ntfp8_gemm_batch(d, len(probs), st)
+        assert rc == 0, rc
+
+    def pcts(v):
+        return {k: round(float(np.percentile(v, p)), 2) for k, p in (("p10", 10), ("p50", 50), ("p90", 90), ("max", 100))}
+
+    def report(n, k_tiles):
+        buf = np.zeros(n * 8, dtype=np.uint64)
+        rc = lib.ntfp8_debug_stamps(buf.ctypes.data, buf.nbytes)
+        assert rc == 0, rc
+        s = buf.reshape(n, 8).astype(np.int64)
+        t = s[:, :5] * 0.01   # 100 MHz ticks -> us
+        t0, t_end = t[:, 0].min(), t[:, 4].max()
+        hw, xcc = s[:, 5] & 0xFFFFFFFF, (s[:, 5] >> 32) & 0xF
+        cycles = (s[:, 7] - s[:, 6]).astype(np.float64)   # shader-clock cycles of the K loop
+        cu = (xcc << 16) | (((hw >> 13) & 7) << 8) | (((hw >> 12) & 1) << 4) | ((hw >> 8) & 0xF)
+        ids = np.unique(cu)
+        handover, idle_end, per_cu = [], [], []
+        for c in ids:
+            idx = np.where(cu == c)[0]
+            idx = idx[np.argsort(t[idx, 0])]
+            per_cu.append(len(idx))
+            idle_end.append(t_end - t[idx[-1], 4])
+            handover += [t[b, 0] - t[a, 4] for a, b in zip(idx, idx[1:])]
+        loop = t[:, 2] - t[:, 1]
+        out = {"workgroups": n, "span_us": round(float(t_end - t0), 1), "cus": int(len(ids)),
+               "workgroups_per_cu": [int(min(per_cu)), int(max(per_cu))],
+               "us_per_workgroup": {"entry_to_first_tile": pcts(t[:, 1] - t[:, 0]), "k_loop": pcts(loop),
+                                    "epilogue_issue": pcts(t[:, 3] - t[:, 2]), "store_drain": pcts(t[:, 4] - t[:, 3]),
+                                    "whole": pcts(t[:, 4] - t[:, 0])},
+               "k_loop_cycles_per_k_tile_p50": round(float(np.median(cycles)) / k_tiles, 1),
+               "k_loop_us_per_k_tile_p50": round(float(np.median(loop)) / k_tiles, 3),
+               "k_loop_shader_clock_ghz_p50": round(float(np.median(cycles / (loop * 1e3))), 3),
+               "cu_idle_before_launch_end_us": pcts(idle_end),
+               "k_loop_p50_by_xcd_us": [round(float(np.median(loop[xcc == k])), 1) for k in range(8)],
+               "last_store_p50_by_xcd_us": [round(float(np.median([t[np.where(cu == c)[0], 4].max() - t0
+                                                                   for c in ids if (c >> 16) == k])), 1) for k in range(8)]}
+        if handover:
+            out["handover_on_a_cu_us"] = pcts(handover)
+        return out
+
+    T = TOKENS
+    x, w = q((T, 4096), 1.0, DTypes.FP8E4M3), q((4096, 4096), 0.02, DTypes.FP8E4M3)
+    w3 = q((12288, 4096), 0.02, DTypes.FP8E4M3)
+    xd, wd = q((T, 14336), 1.0, DTypes.FP8E4M3), q((4096, 14336), 0.02, DTypes.FP8E4M3)
+    gd = q((T, 4096), 1e-3, DTypes.FP8E5M2)
+    y = torch.empty(T, 4096, dtype=torch.bfloat16, device=device)
+    y3 = torch.empty(T, 12288, dtype=torch.bfloat16, device=device)
+    dx = torch.empty(T, 14336, dtype=torch.bfloat16, device=device)
+    dw = torch.empty(4096, 14336, dtype=torch.float32, device=device)
+    bf16, f32 = nt.TORCH_TO_NT[torch.bfloat16], nt.TORCH_TO_NT[torch.float32]
+    pair = [(gd, wd, dx, True, False, bf16), (gd, xd, dw, True, True, f32)]
+    cases = [("o fwd 4096x4096x4096 -> bf16, 1 round", [(x, w, y, False, False, bf16)], 256, 32),
+             ("fwd 4096x12288x4096 -> bf16, 3 rounds", [(x, w3, y3, False, False, bf16)], 768, 32),
+             ("down fwd 4096x4096x14336 -> bf16, 1 round", [(xd, wd, y, False, False, bf16)], 256, 112),
+             ("down dgrad (bf16) + wgrad (fp32), operands read untransposed, 7 rounds", pair, 1792, 32)]
+    res = {}
+    for tag, probs, n, kt in cases:
+        for _ in range(6):
+            run(probs)
+        torch.cuda.synchronize()
+        run(probs)
+        torch.cuda.synchronize()
+        res[tag] = report(n, kt)
+    # the same seven-round launch on a rested chip and under sustained load
+    torch.cuda.synchronize()
+    time.sleep(0.3)
+    run(pair)
+    torch.cuda.synchronize()
+    res["7-round launch, single, after 0.3 s of idle"] = report(1792, 32)
+    for reps in (4, 16):
+        for _ in range(reps):
+            run(pair)
+        torch.cuda.synchronize()
+        res[f"7-round launch, last of {reps} back to back"] = report(1792, 32)
+        time.sleep(0.3)
+    return res
+
+
 def hipblaslt_reference(device, reps=30, nsets=4):
     """The vendor's fp8 GEMM (hipBLASLt behind torch._scaled_mm, e4m3 x e4m3, bf16 output) on the forward shapes of
     the workload, rotating operands as the step does.  A yardstick for the hand-written kernel, not part of the
@@ -621,6 +738,10 @@ def main():
 
     if args.workload == "probe":
         probe(device)
+        return
+    if args.workload == "wg-timeline":
+        print(json.dumps({"workload": "per-workgroup wall-clock stamps inside gemm_nt_big_kernel (profiling build)",
+                          "launches": workgroup_timeline(device)}))
         return
     if args.workload == "vendor-gemm":
         n = args.operand_sets

@@ -1,4 +1,6 @@
-"""Builds nanotron_amd/libntfp8.so (the C-ABI library of include/ntfp8.h) with hipcc for gfx950.
+"""Builds nanotron_amd/libntfp8.so (the C-ABI library of include/ntfp8.h) with hipcc for gfx950, and beside it
+libntfp8_stamps.so, the same library with per-workgroup time stamps compiled into the GEMM kernel (-DNTFP8_STAMPS;
+only `bench.py --workload wg-timeline` loads it).
 
     python -m nanotron_amd.build
 
@@ -15,6 +17,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libntfp8.so")
+LIB_STAMPS = os.path.join(HERE, "libntfp8_stamps.so")
 SOURCES = ["quant.hip", "gemm.hip", "capi.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -25,9 +28,10 @@ FLAGS = [
 ]
 
 
-def _compile(src: str) -> str:
-    obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(job) -> str:
+    src, defines, suffix = job
+    obj = os.path.join(CSRC, src.replace(".hip", suffix + ".o"))
+    cmd = [HIPCC, *FLAGS, *defines, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
@@ -38,11 +42,15 @@ def _compile(src: str) -> str:
 
 
 def build(verbose: bool = True) -> str:
-    with ThreadPoolExecutor(max_workers=len(SOURCES)) as ex:
-        objs = list(ex.map(_compile, SOURCES))
-    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs])
+    jobs = [(s, [], "") for s in SOURCES] + [("gemm.hip", ["-DNTFP8_STAMPS"], "_stamps")]
+    with ThreadPoolExecutor(max_workers=len(jobs)) as ex:
+        objs = list(ex.map(_compile, jobs))
+    plain, stamped = objs[:len(SOURCES)], objs[len(SOURCES)]
+    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *plain])
+    with_stamps = [stamped if o.endswith("gemm.o") else o for o in plain]
+    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_STAMPS, *with_stamps])
     if verbose:
-        print(f"built {LIB}")
+        print(f"built {LIB} and {LIB_STAMPS}")
     return LIB
 
 

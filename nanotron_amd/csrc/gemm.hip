@@ -313,3 +313,12 @@ int run_gemm_batch(const GemmDesc* g, int n, hipStream_t st) {
 }
 
 }  // namespace ntfp8
+
+#ifdef NTFP8_STAMPS
+// Profiling build only: copies the per-workgroup time stamps of the last gemm_nt_big_kernel launches to host memory
+// (8 x uint64 per workgroup index, see gemm_big.h).  Synchronises the device.
+extern "C" __attribute__((visibility("default"))) int ntfp8_debug_stamps(void* dst, size_t bytes) {
+    if (!dst || bytes > sizeof(unsigned long long) * ntfp8::kStampSlots * 8) return dst ? NTFP8_ERR_SIZE : NTFP8_ERR_NULL;
+    return hipMemcpyFromSymbol(dst, HIP_SYMBOL(ntfp8::g_stamps), bytes) == hipSuccess ? NTFP8_OK : NTFP8_ERR_LAUNCH;
+}
+#endif

@@ -26,6 +26,21 @@
 
 namespace ntfp8 {
 
+// Profiling build (-DNTFP8_STAMPS, libntfp8_stamps.so): every workgroup of gemm_nt_big_kernel leaves five readings of
+// the 100 MHz wall clock (kernel entry, first tile published, end of the K loop, last store issued, stores drained), the
+// shader-clock cycle counter at both ends of the K loop and the identity of its CU in a table that
+// ntfp8_debug_stamps() copies out.  The product library is built without it.
+#ifdef NTFP8_STAMPS
+constexpr int kStampSlots = 16384;
+__device__ unsigned long long g_stamps[kStampSlots * 8];
+#define NTFP8_STAMP(var) var = wall_clock64()
+#define NTFP8_CYCLES(var) var = __builtin_readcyclecounter()
+#else
+#define NTFP8_STAMP(var) (void)0
+#define NTFP8_CYCLES(var) (void)0
+#endif
+
+
 constexpr int kBigN = 256;
 constexpr int kBigWaves = 4, kBigThreads = kBigWaves * 64;
 constexpr int kBigNJ = 8;              // 16-column accumulator blocks per wave: 128 columns
@@ -279,6 +294,8 @@ void gemm_nt_big_kernel(const BigLaunch L) {
     __shared__ __attribute__((aligned(1024))) uint8_t sB[NS][kBigN * kBK];
 
     // ---- which tile (or half tile) of which problem is this workgroup's ----------------------------
+    [[maybe_unused]] unsigned long long st_entry = 0, st_first = 0, st_loop = 0, cy_first = 0, cy_loop = 0;
+    NTFP8_STAMP(st_entry);
     int pid = blockIdx.x;
     int half = 0;
     if constexpr (MI == 8) {
@@ -601,6 +618,8 @@ void gemm_nt_big_kernel(const BigLaunch L) {
             for (int l = 0; l < NL; ++l) issue(1, l);
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");   // tile 0 has landed, tile 1 may still be in flight
             wg_barrier();
+            NTFP8_STAMP(st_first);
+            NTFP8_CYCLES(cy_first);
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
                 fa[i][0] = rd_a(0, i, 0);
@@ -689,6 +708,8 @@ void gemm_nt_big_kernel(const BigLaunch L) {
         kloop(std::false_type{});
     }
 
+    NTFP8_STAMP(st_loop);
+    NTFP8_CYCLES(cy_loop);
     {
         // output type, accumulation and bias are properties of the problem, not of the kernel (fp8 outputs apart)
         auto epilogue = [&](auto bias_tag, const float (*bv)[4]) {
@@ -725,6 +746,21 @@ void gemm_nt_big_kernel(const BigLaunch L) {
             epilogue(std::false_type{}, nullptr);
         }
     }
+#ifdef NTFP8_STAMPS
+    {
+        const unsigned long long st_issued = wall_clock64();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const unsigned long long st_drained = wall_clock64();
+        if (threadIdx.x == 0) {
+            unsigned long long* o = g_stamps + (size_t)(blockIdx.x % kStampSlots) * 8;
+            o[0] = st_entry, o[1] = st_first, o[2] = st_loop, o[3] = st_issued, o[4] = st_drained;
+            // HW_ID (cu 11:8, sh 12, se 15:13) | XCC_ID << 32 | MI << 40
+            o[5] = (unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 4) |
+                   ((unsigned long long)(__builtin_amdgcn_s_getreg((31 << 11) | 20) & 0xf) << 32) | ((unsigned long long)MI << 40);
+            o[6] = cy_first, o[7] = cy_loop;
+        }
+    }
+#endif
 }
 
 }  // namespace ntfp8
