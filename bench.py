@@ -637,6 +637,19 @@ def workgroup_timeline(device):
         run(probs)
         torch.cuda.synchronize()
         res[tag] = report(n, kt)
+    # what the fetch traffic costs: the same launches with the XCD-aware tile order switched off (every XCD then pulls
+    # every operand panel through its own L2)
+    lib.ntfp8_debug_set_tile_order.restype = ctypes.c_int
+    lib.ntfp8_debug_set_tile_order.argtypes = [ctypes.c_int]
+    for tag, probs, n, kt in cases[1:3]:
+        for plain in (1, 0):
+            assert lib.ntfp8_debug_set_tile_order(plain) == 0
+            for _ in range(6):
+                run(probs)
+            torch.cuda.synchronize()
+            run(probs)
+            torch.cuda.synchronize()
+            res[tag + (" | tiles in launch order" if plain else " | XCD-aware order (repeat)")] = report(n, kt)
     # the same seven-round launch on a rested chip and under sustained load
     torch.cuda.synchronize()
     time.sleep(0.3)

@@ -321,4 +321,8 @@ extern "C" __attribute__((visibility("default"))) int ntfp8_debug_stamps(void* d
     if (!dst || bytes > sizeof(unsigned long long) * ntfp8::kStampSlots * 8) return dst ? NTFP8_ERR_SIZE : NTFP8_ERR_NULL;
     return hipMemcpyFromSymbol(dst, HIP_SYMBOL(ntfp8::g_stamps), bytes) == hipSuccess ? NTFP8_OK : NTFP8_ERR_LAUNCH;
 }
+extern "C" __attribute__((visibility("default"))) int ntfp8_debug_set_tile_order(int plain) {
+    const int v = plain ? 1 : 0;
+    return hipMemcpyToSymbol(HIP_SYMBOL(ntfp8::g_plain_tile_order), &v, sizeof(v)) == hipSuccess ? NTFP8_OK : NTFP8_ERR_LAUNCH;
+}
 #endif

@@ -33,6 +33,9 @@ namespace ntfp8 {
 #ifdef NTFP8_STAMPS
 constexpr int kStampSlots = 16384;
 __device__ unsigned long long g_stamps[kStampSlots * 8];
+// 1: workgroups take the tiles in launch order, i.e. every XCD gets every eighth tile and touches all operand panels
+// (an experiment on what the fetch traffic costs; set with ntfp8_debug_set_tile_order)
+__device__ int g_plain_tile_order = 0;
 #define NTFP8_STAMP(var) var = wall_clock64()
 #define NTFP8_CYCLES(var) var = __builtin_readcyclecounter()
 #else
@@ -305,6 +308,10 @@ void gemm_nt_big_kernel(const BigLaunch L) {
         const int round0 = (pid / L.round_size) * L.round_size;
         const int in_round = min(L.round_size, L.full_blocks - round0);
         const int local = pid - round0;
+#ifdef NTFP8_STAMPS
+        if (g_plain_tile_order) {
+        } else
+#endif
         if (in_round % kXcds == 0) pid = round0 + (local % kXcds) * (in_round / kXcds) + local / kXcds;
     } else {
         const int nb = 2 * L.tail_tiles;
