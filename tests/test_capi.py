@@ -304,3 +304,72 @@ def test_static_scratch_entry_point_rejects_what_it_cannot_hold():
     assert L.ntfp8_quantize_delayed_batch_static(one(desc(0, out=P + 8)), 1, None) == -7
     two = (nt.QuantDesc * 2)(desc(0), desc(1, amax_out=P + 8192))
     assert L.ntfp8_quantize_delayed_batch_static(two, 2, None) == -7
+
+
+def test_tex_shim_rejects_what_it_does_not_serve_before_touching_the_gpu():
+    """The Transformer-Engine-shaped binding raises RuntimeError (TE's C++ exceptions surface as that) for the forms
+    it does not serve and for host tensors; no GPU is needed to get these answers."""
+    import torch
+
+    from nanotron_amd import tex_shim as tex
+
+    e = torch.empty(0)
+    a = torch.zeros(32, 32, dtype=torch.uint8)
+    one = torch.ones(1)
+    D = torch.empty(32, 32)
+
+    def gemm(**kw):
+        args = dict(A=a, A_scale_inverse=one, A_type=tex.DType.kFloat8E4M3, transa=True, B=a, B_scale_inverse=one,
+                    B_type=tex.DType.kFloat8E4M3, transb=False, D=D, D_scale=e, D_type=tex.DType.kFloat32, D_amax=e,
+                    bias=e, bias_type=tex.DType.kBFloat16, pre_gelu_out=e, grad=False, workspace=e, workspaceSize=0,
+                    accumulate=False, use_split_accumulator=False, math_sm_count=0)
+        args.update(kw)
+        return tex.te_gemm(*args.values())
+
+    with pytest.raises(RuntimeError, match="transa=True with transb=True"):
+        gemm(transb=True)
+    with pytest.raises(RuntimeError, match="GELU"):
+        gemm(pre_gelu_out=torch.zeros(4))
+    with pytest.raises(RuntimeError, match="bias-gradient"):
+        gemm(grad=True, bias=torch.zeros(32))
+    with pytest.raises(RuntimeError, match="2-D"):
+        gemm(A=torch.zeros(32, dtype=torch.uint8))
+    with pytest.raises(RuntimeError, match="reduction lengths"):
+        gemm(B=torch.zeros(32, 48, dtype=torch.uint8))
+    with pytest.raises(RuntimeError, match="device tensor"):
+        tex.cast_to_fp8(torch.zeros(4, 4), one, one.clone(), one.clone(), tex.DType.kFloat8E4M3)
+    with pytest.raises(RuntimeError, match="device tensor"):
+        tex.cast_from_fp8(a, one, tex.DType.kFloat8E4M3, tex.DType.kFloat32)
+    with pytest.raises(RuntimeError, match="not an FP8 type"):
+        tex.fp8_transpose(a, tex.DType.kFloat32)
+    # install() registers the module under the names the reference imports
+    import sys
+    keep = {k: sys.modules.get(k) for k in ("transformer_engine", "transformer_engine_extensions")}
+    try:
+        assert tex.install() is tex and sys.modules["transformer_engine_extensions"] is tex
+        assert "transformer_engine" in sys.modules
+    finally:
+        for k, v in keep.items():
+            if v is None:
+                sys.modules.pop(k, None)
+            else:
+                sys.modules[k] = v
+
+
+def test_profiling_build_exports_its_accessors():
+    """libntfp8_stamps.so (the GEMM compiled with -DNTFP8_STAMPS, loaded only by bench.py --workload wg-timeline) is
+    the product library plus two accessors; the product library does not carry them."""
+    import ctypes
+    import os
+
+    from nanotron_amd import _native as nt
+
+    path = os.path.join(os.path.dirname(nt.__file__), "libntfp8_stamps.so")
+    assert os.path.exists(path), "python -m nanotron_amd.build builds it"
+    lib = ctypes.CDLL(path)
+    for name in ("ntfp8_debug_stamps", "ntfp8_debug_set_tile_order", "ntfp8_gemm_batch", "ntfp8_version"):
+        assert hasattr(lib, name), name
+    assert not hasattr(nt.lib, "ntfp8_debug_stamps")
+    lib.ntfp8_debug_stamps.restype = ctypes.c_int
+    lib.ntfp8_debug_stamps.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+    assert lib.ntfp8_debug_stamps(None, 64) == nt.ERR_NULL if hasattr(nt, "ERR_NULL") else lib.ntfp8_debug_stamps(None, 64) < 0
