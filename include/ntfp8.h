@@ -195,7 +195,8 @@ typedef struct ntfp8_gemm_desc {
      * reduces over N_out; wgrad: X[tokens, K_in] reduces over tokens; src/nanotron/fp8/linear.py:104-109), and
      * where the reference calls tex.fp8_transpose first (src/nanotron/fp8/kernel.py:43) this library reads the
      * tensor as it is.  Served for N a multiple of 16, M and N above 128, K at least 256, operands below 2 GiB
-     * and outputs other than fp8; anything else returns NTFP8_ERR_UNSUPPORTED (transpose B and pass 0). */
+     * (fp8 outputs in addition: M a multiple of 4, M N below 2^32, D_t aligned to 16 bytes); anything else returns
+     * NTFP8_ERR_UNSUPPORTED (transpose B and pass 0). */
     int b_transposed;
     /* NULL, or bias[N] of type bias_dtype (NTFP8_F32 / NTFP8_F16 / NTFP8_BF16), added to the descaled fp32 result
      * before the single rounding to d_dtype: D = round(fp32(acc * descale) + bias[n]).  This is the `bias` /

@@ -88,7 +88,6 @@ int check_gemm(const ntfp8_gemm_desc& p, GemmDesc* g) {
                   nullptr, nullptr, nullptr, p.b_transposed ? 1 : 0, p.bias, p.bias ? p.bias_dtype : NTFP8_F32,
                   p.scales_are_inverse ? 1 : 0, p.a_transposed ? 1 : 0};
     if (p.a_transposed && !p.b_transposed) return NTFP8_ERR_UNSUPPORTED;
-    if (p.b_transposed && fp8_out) return NTFP8_ERR_UNSUPPORTED;
     if (fp8_out) {
         if (!is_aligned(p.scale_d, 4) || (p.amax_workspace && !is_aligned(p.amax_workspace, 4))) return NTFP8_ERR_ALIGN;
         if (p.D_t && (overlap(p.A, (size_t)mk, p.D_t, db) || overlap(p.B, (size_t)nk, p.D_t, db) || overlap(p.D, db, p.D_t, db)))

@@ -183,7 +183,7 @@ static int path_of(const GemmDesc& g) {
     // an operand given as its transpose, [K, N] or [K, M], is loaded in 16-byte pieces of its rows; only the big
     // kernel reads it, and a transposed A only next to a transposed B (the wgrad form)
     if (g.ta && (!g.tb || g.M % 16 != 0)) return kPathNone;
-    if (g.tb) return (g.N % 16 == 0 && fits32 && worth && !is_fp8_out(g.d_dtype)) ? kPathBig : kPathNone;
+    if (g.tb) return (g.N % 16 == 0 && fits32 && worth && fp8_ok) ? kPathBig : kPathNone;
     return (fits32 && worth && fp8_ok) ? kPathBig : kPathSmall;
 }
 
@@ -259,7 +259,8 @@ template <int FA, int FB>
 static int dispatch_fmt(const GemmDesc* const* g, int n, int path, hipStream_t st) {
     if (path == kPathNone) return NTFP8_ERR_UNSUPPORTED;
     if (path == kPathBig) {
-        if (g[0]->tb) return launch_big<FA, FB, false, true>(g, n, st);
+        if (g[0]->tb)
+            return is_fp8_out(g[0]->d_dtype) ? launch_big<FA, FB, true, true>(g, n, st) : launch_big<FA, FB, false, true>(g, n, st);
         return is_fp8_out(g[0]->d_dtype) ? launch_big<FA, FB, true, false>(g, n, st) : launch_big<FA, FB, false, false>(g, n, st);
     }
     const GemmDesc& d = *g[0];   // the small kernels take one problem

@@ -192,11 +192,15 @@ __device__ __forceinline__ void reg_store4(__amdgpu_buffer_rsrc_t r, uint32_t vo
 // All stores go through buffer descriptors of M N bytes: rows past the end fall outside and are dropped, columns
 // past the end get an offset that does; nothing is predicated, which keeps the scalar registers of the epilogue
 // (and with them the register budget of the K loop before it) small.
-template <int F, int MI, int NJ, bool kBias = false>
+// kMask: accumulator blocks past N (and past M if `mask_rows`: A given as its transpose) hold arbitrary values,
+// because an operand read through the transposing loads wraps into its next row there instead of reading zeros, and
+// must stay out of the amax.  N (and M, with a transposed A) is a multiple of 16 then, so whole blocks are in or
+// out, uniformly for the wave.  Rows past M of an ordinary A operand read as zeros and need no mask.
+template <int F, int MI, int NJ, bool kBias = false, bool kMask = false>
 __device__ __forceinline__ uint32_t store_wave_tile16_fp8(const v4f (&acc)[MI][NJ], uint8_t* __restrict__ D,
                                                           uint8_t* __restrict__ Dt, float alpha, float scale_d, bool slow,
                                                           int M, int N, int m_base, int n_base, int lane,
-                                                          const float (*bv)[4] = nullptr) {
+                                                          const float (*bv)[4] = nullptr, bool mask_rows = false) {
     auto val = [&](int i, int j, int e) -> float {
         if constexpr (kBias) return acc[i][j][e] * alpha + bv[j][e];
         else return acc[i][j][e] * alpha;
@@ -214,8 +218,15 @@ __device__ __forceinline__ uint32_t store_wave_tile16_fp8(const v4f (&acc)[MI][N
         const int mq = m & ~3;
         uint32_t w[NJ];
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
-            w[j] = quant4<F>(val(i, j, 0), val(i, j, 1), val(i, j, 2), val(i, j, 3), scale_d, slow, amax);
+        for (int j = 0; j < NJ; ++j) {
+            if constexpr (kMask) {
+                uint32_t a = amax;
+                w[j] = quant4<F>(val(i, j, 0), val(i, j, 1), val(i, j, 2), val(i, j, 3), scale_d, slow, a);
+                if ((!mask_rows || m_base + i * 16 < M) && n_base + j * 16 < N) amax = a;
+            } else {
+                w[j] = quant4<F>(val(i, j, 0), val(i, j, 1), val(i, j, 2), val(i, j, 3), scale_d, slow, amax);
+            }
+        }
         if (Dt) {   // uniform
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
@@ -726,10 +737,10 @@ void gemm_nt_big_kernel(const BigLaunch L) {
                 const bool slow = scale_is_degenerate(scale_d);
                 const uint32_t amax =
                     P.d_dtype == NTFP8_OUT_E4M3
-                        ? store_wave_tile16_fp8<kE4M3, MI, kBigNJ, kBias>(acc, static_cast<uint8_t*>(Dv), P.fp8.Dt, alpha, scale_d,
-                                                                          slow, M, N, m0 + wm, n0 + wn, lane, bv)
-                        : store_wave_tile16_fp8<kE5M2, MI, kBigNJ, kBias>(acc, static_cast<uint8_t*>(Dv), P.fp8.Dt, alpha, scale_d,
-                                                                          slow, M, N, m0 + wm, n0 + wn, lane, bv);
+                        ? store_wave_tile16_fp8<kE4M3, MI, kBigNJ, kBias, kBT>(acc, static_cast<uint8_t*>(Dv), P.fp8.Dt, alpha, scale_d,
+                                                                          slow, M, N, m0 + wm, n0 + wn, lane, bv, kBT && P.at)
+                        : store_wave_tile16_fp8<kE5M2, MI, kBigNJ, kBias, kBT>(acc, static_cast<uint8_t*>(Dv), P.fp8.Dt, alpha, scale_d,
+                                                                          slow, M, N, m0 + wm, n0 + wn, lane, bv, kBT && P.at);
                 publish_amax(amax, P.fp8.ws);
             } else if (P.d_dtype == NTFP8_BF16) {
                 store_wave_tile16<NTFP8_BF16, false, MI, kBigNJ, kBias>(acc, Dv, alpha, M, N, m0 + wm, n0 + wn, lane, bv);

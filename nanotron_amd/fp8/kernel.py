@@ -51,7 +51,7 @@ def _gemm_nt(a: FP8Tensor, b: FP8Tensor, out_dtype: torch.dtype, accumulate_into
 
 
 def _gemm_nt_fp8(a: FP8Tensor, b: FP8Tensor, dtype: DTypes, state: Optional[DelayedScaling],
-                 with_transpose: bool, bias: Optional[torch.Tensor] = None) -> FP8Tensor:
+                 with_transpose: bool, bias: Optional[torch.Tensor] = None, bt: bool = False, at: bool = False) -> FP8Tensor:
     """FP8Tensor(_gemm_nt(a, b, float32), dtype, state=state, with_transpose=with_transpose), bit for bit, with the
     fp32 result never written to memory: the GEMM epilogue casts with the scale `state` holds from earlier steps,
     leaves max|result| behind, and a one-wave kernel turns that into amax, history roll and next scale.
@@ -62,11 +62,16 @@ def _gemm_nt_fp8(a: FP8Tensor, b: FP8Tensor, dtype: DTypes, state: Optional[Dela
 
     assert dtype in _OUT_FMT, f"{dtype} is not an FP8 format"
     if state is None or not state.initialised:
-        return FP8Tensor(_gemm_nt(a, b, torch.float32, None, bias), dtype, state=state, with_transpose=with_transpose)
+        hp = (_gemm_nt_batch([(a, b, torch.float32, None, True, None, at)])[0] if bt
+              else _gemm_nt(a, b, torch.float32, None, bias))
+        return FP8Tensor(hp, dtype, state=state, with_transpose=with_transpose)
     assert state.dtype == dtype, "delayed-scaling state was created for another format"
-    assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[1], (tuple(a.shape), tuple(b.shape))
-    M, K = a.shape
-    N = b.shape[0]
+    assert a.dim() == 2 and b.dim() == 2 and a.shape[0 if at else 1] == b.shape[0 if bt else 1], \
+        (tuple(a.shape), tuple(b.shape), bt, at)
+    assert not at or bt, "a transposed A operand is only read next to a transposed B operand"
+    assert bias is None or not bt, "no bias together with a transposed B operand"
+    K, M = a.shape if at else a.shape[::-1]
+    N = b.shape[1 if bt else 0]
     dev = a.device
     assert state._buf.device == dev
     a, ma = _bytes_and_meta(a)
@@ -84,6 +89,7 @@ def _gemm_nt_fp8(a: FP8Tensor, b: FP8Tensor, dtype: DTypes, state: Optional[Dela
     d[0].M, d[0].N, d[0].K = M, N, K
     d[0].fmt_a, d[0].fmt_b, d[0].d_dtype, d[0].accumulate = _FMT[ma.dtype], _FMT[mb.dtype], _OUT_FMT[dtype], 0
     d[0].scale_d, d[0].D_t, d[0].amax_workspace = state_p, nt.ptr(out_t), ws.data_ptr()
+    d[0].b_transposed, d[0].a_transposed = int(bt), int(at)
     if bias is not None:
         d[0].bias, d[0].bias_dtype = bias.data_ptr(), nt.TORCH_TO_NT[bias.dtype]
     nt.check(nt.lib.ntfp8_gemm_batch(d, 1, st), "ntfp8_gemm_batch")
@@ -245,9 +251,10 @@ def fp8_matmul_kernel(
     assert hasattr(mat_a, "fp8_meta") and hasattr(mat_b, "fp8_meta"), "operands must be FP8Tensors"
     if isinstance(out_dtype, DTypes):
         assert accumulate_into is None, "an fp8 output cannot accumulate"
-        a_ = mat_a if transpose_a else mat_a.transposed()  # kernel.py:43
-        b_ = mat_b.transposed() if transpose_b else mat_b  # kernel.py:44
-        return _gemm_nt_fp8(b_, a_, out_dtype, out_state, out_with_transpose, bias)
+        # rows of D: the fp8 epilogue stores whole words of 4 rows' worth of the transposed copy
+        rows = mat_b.shape[1] if transpose_b else mat_b.shape[0]
+        A, B, bt, at = _operands(mat_a, transpose_a, mat_b, transpose_b, None, allow_bt=bias is None and rows % 4 == 0)
+        return _gemm_nt_fp8(A, B, out_dtype, out_state, out_with_transpose, bias, bt, at)
     A, B, bt, at = _operands(mat_a, transpose_a, mat_b, transpose_b, accumulate_into, allow_bt=bias is None)
     if bt:
         return _gemm_nt_batch([(A, B, out_dtype or torch.float32, accumulate_into, True, None, at)])[0]

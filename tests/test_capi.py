@@ -160,7 +160,8 @@ def test_fp8_output_and_transposed_operand_requests_are_validated_before_any_lau
     assert L.ntfp8_gemm_batch(desc(d_dtype=nt.OUT_E5M2, scale_d=P + (4 << 20), accumulate=1), 1, None) == -5
     assert L.ntfp8_gemm_batch(desc(d_dtype=nt.OUT_E4M3, scale_d=P + (4 << 20) + 2), 1, None) == -4        # misaligned scale
     assert L.ntfp8_gemm_batch(desc(d_dtype=nt.OUT_E4M3, scale_d=P + (4 << 20), D_t=P + (3 << 20) + 64), 1, None) == -7
-    assert L.ntfp8_gemm_batch(desc(d_dtype=nt.OUT_E4M3, scale_d=P + (4 << 20), b_transposed=1), 1, None) == -5
+    # an fp8 output next to a transposed B operand is served for M a multiple of 4 only (whole words of the transposed copy)
+    assert L.ntfp8_gemm_batch(desc(M=254, d_dtype=nt.OUT_E4M3, scale_d=P + (4 << 20), b_transposed=1), 1, None) == -5
     assert L.ntfp8_gemm_batch(desc(d_dtype=7), 1, None) == -2
     assert L.ntfp8_gemm(P, 0, P + (1 << 20), P + (2 << 20), 0, P + (1 << 20), P + (3 << 20), nt.OUT_E4M3, 256, 256, 256, 0, None) == -5
     # a transposed B operand outside what the kernels serve

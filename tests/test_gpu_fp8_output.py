@@ -225,6 +225,54 @@ def test_two_linears_chained_through_an_fp8_activation():
     assert "fp8_state.output" in first.state_dict()
 
 
+@pytest.mark.parametrize("fo", FMTS)
+@pytest.mark.parametrize("form", ["dgrad", "wgrad"])
+@pytest.mark.parametrize("shape", [(512, 384, 640), (4096, 1024, 2048), (272, 400, 288)])
+def test_fp8_output_with_operands_read_untransposed_equals_the_materialised_transposes(fo, form, shape):
+    """An fp8 output next to `b_transposed` (dgrad form) and `a_transposed` + `b_transposed` (wgrad form): bytes,
+    transposed bytes, amax, scale and history equal those of the same GEMM on transposed copies, bit for bit, and both
+    equal the two-step form (fp32 GEMM, then the delayed-scaling cast)."""
+    import nanotron_amd.fp8.kernel as K
+    from nanotron_amd.fp8 import FP8Tensor
+    from nanotron_amd.fp8.kernel import fp8_matmul_kernel
+
+    T, n_out, k_in = shape
+    gy = FP8Tensor(O.normal_tensor(11, (T, n_out), 1e-2, torch.bfloat16).cuda(), _dt(O.E5M2))
+    w = FP8Tensor(O.normal_tensor(12, (n_out, k_in), 0.05, torch.bfloat16).cuda(), _dt(O.E4M3))
+    x = FP8Tensor(O.normal_tensor(13, (T, k_in), 1.0, torch.bfloat16).cuda(), _dt(O.E4M3))
+    if form == "dgrad":     # dX[T, k_in] = dY . W        (linear.py:104-106)
+        args = dict(mat_a=w, transpose_a=False, mat_b=gy, transpose_b=False)
+    else:                   # dW[n_out, k_in] = dY^T . X  (linear.py:107-109)
+        args = dict(mat_a=x, transpose_a=False, mat_b=gy, transpose_b=True)
+    st0 = _state_with_scale(fo, 64.0, history_len=4, hist=[0.5, 0.25, 2.0, 1.0])
+    res = {}
+    for mode in ("as_is", "copies"):
+        K.READ_B_TRANSPOSED = K.READ_A_TRANSPOSED = mode == "as_is"
+        try:
+            for t in (gy, w, x):
+                t._transposed = None
+            st = _clone_state(st0)
+            A, B, bt, at = K._operands(args["mat_a"], False, args["mat_b"], args["transpose_b"], None)
+            assert (bt, at) == ((True, form == "wgrad") if mode == "as_is" else (False, False))
+            for t in (gy, w, x):
+                t._transposed = None
+            out = fp8_matmul_kernel(**args, use_split_accumulator=False, out_dtype=_dt(fo), out_state=st, out_with_transpose=True)
+            res[mode] = (out, st)
+        finally:
+            K.READ_B_TRANSPOSED = K.READ_A_TRANSPOSED = True
+    (o1, s1), (o2, s2) = res["as_is"], res["copies"]
+    assert torch.equal(o1.as_subclass(torch.Tensor), o2.as_subclass(torch.Tensor))
+    assert torch.equal(o1._transposed.as_subclass(torch.Tensor), o2._transposed.as_subclass(torch.Tensor))
+    assert torch.equal(o1._transposed.as_subclass(torch.Tensor), o1.as_subclass(torch.Tensor).t().contiguous())
+    assert _same_f32(o1.fp8_meta.amax, o2.fp8_meta.amax) and _same_f32(o1.fp8_meta.scale, o2.fp8_meta.scale)
+    assert _same_f32(s1._buf, s2._buf)
+    # the two-step form on the fp32 result of the same kernel
+    hp = fp8_matmul_kernel(**args, use_split_accumulator=False)
+    two = FP8Tensor(hp, _dt(fo), state=_clone_state(st0))
+    assert torch.equal(o1.as_subclass(torch.Tensor), two.as_subclass(torch.Tensor))
+    assert _same_f32(o1.fp8_meta.amax, two.fp8_meta.amax)
+
+
 def test_batch_mixes_fp8_and_plain_outputs_and_rejects_bad_requests():
     from nanotron_amd import _native as nt
     from nanotron_amd.fp8 import FP8Tensor

@@ -135,7 +135,8 @@ def test_requests_the_kernels_do_not_serve_are_refused():
     for M, N, K in [(256, 250, 256), (128, 256, 256), (256, 128, 256), (256, 256, 128), (256, 256, 250)]:
         assert not b_transposed_supported(M, N, K)
         assert call(M, N, K) == unsupported, (M, N, K)
-    assert call(256, 256, 256, nt.OUT_E4M3, torch.ones(1, device=dev)) == unsupported   # no fp8 output from this kernel
+    assert call(256, 256, 256, nt.OUT_E4M3, torch.ones(1, device=dev)) == 0              # fp8 outputs are served ...
+    assert call(254, 256, 256, nt.OUT_E4M3, torch.ones(1, device=dev)) == unsupported    # ... for M a multiple of 4
 
 
 @pytest.mark.parametrize("master", [torch.float32, torch.bfloat16])
