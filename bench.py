@@ -629,6 +629,10 @@ def workgroup_timeline(device):
              ("fwd 4096x12288x4096 -> bf16, 3 rounds", [(x, w3, y3, False, False, bf16)], 768, 32),
              ("down fwd 4096x4096x14336 -> bf16, 1 round", [(xd, wd, y, False, False, bf16)], 256, 112),
              ("down dgrad (bf16) + wgrad (fp32), operands read untransposed, 7 rounds", pair, 1792, 32)]
+    wh = q((2048, 4096), 0.02, DTypes.FP8E4M3)
+    yh = torch.empty(T, 2048, dtype=torch.bfloat16, device=device)
+    cases.append(("fwd 4096x2048x4096 -> bf16, 128 tiles as 256 half tiles (the tail kernel alone)",
+                  [(x, wh, yh, False, False, bf16)], 256, 32))
     res = {}
     for tag, probs, n, kt in cases:
         for _ in range(6):

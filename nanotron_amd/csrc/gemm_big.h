@@ -692,6 +692,8 @@ void gemm_nt_big_kernel(const BigLaunch L) {
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
         }
         wg_barrier();
+        NTFP8_STAMP(st_first);
+        NTFP8_CYCLES(cy_first);
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
             fa[i][0] = rd_a(0, i, 0);
