@@ -343,3 +343,53 @@ def test_fp8_output_without_consumer_gradient_and_with_two_consumers():
     with torch.no_grad():
         h = l1(x)
         assert l2(h).shape == (160, 128)
+
+
+# ------------------------------------------------------------------------------------------ overlapping streams
+def test_quantisations_on_two_streams_at_once_equal_the_serial_results():
+    """Calls that may overlap in time must use different reduction workspaces; the Python layer keeps one per (device,
+    stream).  Two streams quantise different tensors over and over without waiting for each other: every result equals
+    the one computed alone, bit for bit, and both workspaces are left zero."""
+    from nanotron_amd import _native as nt
+    from nanotron_amd.fp8 import DelayedScaling, DTypes, FP8Tensor
+
+    dev = torch.device("cuda", 0)
+    xs = [O.normal_tensor(40 + i, (2048, 4096), 10.0 ** (i - 2), torch.bfloat16).cuda() for i in range(4)]
+    fmts = [DTypes.FP8E4M3, DTypes.FP8E5M2, DTypes.FP8E4M3, DTypes.FP8E5M2]
+
+    def run(i, steps, out):
+        st = DelayedScaling(fmts[i], 16, 0, dev)
+        for s in range(steps):
+            q = FP8Tensor(xs[(i + s) % 4], fmts[i], state=st)
+            out.append((q.as_subclass(torch.Tensor).clone(), q.fp8_meta.amax.clone(), q.fp8_meta.scale.clone(), st._buf.clone()))
+
+    serial = [[], []]
+    for i in (0, 1):
+        run(i, 12, serial[i])
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    both = [[], []]
+    for s in streams:
+        s.wait_stream(torch.cuda.current_stream())
+    # the first quantisation of a role reads a flag on the host; interleave call by call so that the streams' kernels
+    # are queued side by side
+    states = [DelayedScaling(fmts[i], 16, 0, dev) for i in (0, 1)]
+    for step in range(12):
+        for i in (0, 1):
+            with torch.cuda.stream(streams[i]):
+                q = FP8Tensor(xs[(i + step) % 4], fmts[i], state=states[i])
+                both[i].append((q.as_subclass(torch.Tensor).clone(), q.fp8_meta.amax.clone(), q.fp8_meta.scale.clone(),
+                                states[i]._buf.clone()))
+    torch.cuda.synchronize()
+    for i in (0, 1):
+        for step, (a, b) in enumerate(zip(serial[i], both[i])):
+            assert torch.equal(a[0], b[0]), (i, step)
+            for u, v in zip(a[1:], b[1:]):
+                assert torch.equal(u.view(-1).view(torch.int32), v.view(-1).view(torch.int32)), (i, step)
+    w0 = nt.workspace_and_stream(dev)[0]
+    with torch.cuda.stream(streams[0]):
+        w1 = nt.workspace_and_stream(dev)[0]
+    with torch.cuda.stream(streams[1]):
+        w2 = nt.workspace_and_stream(dev)[0]
+    assert len({w0.data_ptr(), w1.data_ptr(), w2.data_ptr()}) == 3
+    assert int(w1.view(torch.int32).abs().sum()) == 0 and int(w2.view(torch.int32).abs().sum()) == 0
