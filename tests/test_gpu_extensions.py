@@ -393,3 +393,68 @@ def test_quantisations_on_two_streams_at_once_equal_the_serial_results():
         w2 = nt.workspace_and_stream(dev)[0]
     assert len({w0.data_ptr(), w1.data_ptr(), w2.data_ptr()}) == 3
     assert int(w1.view(torch.int32).abs().sum()) == 0 and int(w2.view(torch.int32).abs().sum()) == 0
+
+
+# ------------------------------------------------------------------------------------------ beyond 2^31
+def test_quantisation_of_more_than_two_to_the_31_elements():
+    """Element counts are 64-bit end to end: a bf16 tensor of 2^31 + 12288 elements (4 GiB) is quantised with current
+    scaling; the amax is found wherever it lies, the bytes at both ends equal the oracle's, the zeros in between
+    stay zero."""
+    from nanotron_amd.fp8 import DTypes, FP8Tensor
+
+    n = (1 << 31) + 12288
+    edge = 1 << 20
+    x = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
+    head = O.normal_tensor(71, (edge,), 1.0, torch.bfloat16)
+    tail = O.normal_tensor(72, (edge,), 1.0, torch.bfloat16)
+    x[:edge] = head.cuda()
+    x[-edge:] = tail.cuda()
+    x[(1 << 31) + 7] = -6.5          # the maximum lies behind the 2^31-th element
+    tail[edge - 12288 + 7] = -6.5
+    q = FP8Tensor(x, DTypes.FP8E4M3)
+    assert float(q.fp8_meta.amax) == 6.5
+    scale = q.fp8_meta.scale.cpu()
+    assert float(scale) == float(O.update_scaling_factor(torch.tensor(6.5), torch.tensor(1.0), O.E4M3))
+    raw = q.as_subclass(torch.Tensor)
+    assert raw.shape == (n,)
+    assert torch.equal(raw[:edge].cpu(), O.cast_to_fp8(head, scale, O.E4M3))
+    assert torch.equal(raw[-edge:].cpu(), O.cast_to_fp8(tail, scale, O.E4M3))
+    for lo in (edge, 1 << 30, (1 << 31) - (1 << 23)):
+        assert int(raw[lo:lo + (1 << 22)].to(torch.int32).sum()) == 0
+    del x, q, raw
+    torch.cuda.empty_cache()
+
+
+def test_gemm_with_an_operand_of_more_than_2_gib():
+    """An A operand of 33024 x 65536 bytes does not fit the 32-bit buffer offsets of the 256-tile kernel; the library
+    sends it to the kernel that addresses with 64-bit pointers.  Integer-valued operands: every output must be exact."""
+    from nanotron_amd.fp8 import DTypes, FP8Tensor
+    from nanotron_amd.fp8.kernel import _gemm_nt
+    from nanotron_amd.fp8.meta import FP8Meta
+
+    dev = torch.device("cuda", 0)
+    M, N, K = 33024, 192, 65536
+    codes = torch.tensor([0x00, 0x38, 0x40, 0xB8, 0xC0], dtype=torch.uint8, device=dev)   # 0, 1, 2, -1, -2 in e4m3
+    vals = torch.tensor([0.0, 1.0, 2.0, -1.0, -2.0], device=dev)
+    g = torch.Generator(device=dev).manual_seed(5)
+    ia = torch.randint(0, 5, (M, K), generator=g, device=dev, dtype=torch.uint8)
+    ib = torch.randint(0, 5, (N, K), generator=g, device=dev, dtype=torch.uint8)
+
+    def fp8(idx):
+        t = torch.Tensor._make_subclass(FP8Tensor, codes[idx.long()] if idx.numel() < (1 << 28) else _lookup(idx))
+        t.fp8_meta = FP8Meta(torch.tensor(2.0, device=dev), torch.tensor(1.0, device=dev), DTypes.FP8E4M3)
+        return t
+
+    def _lookup(idx):   # row blocks, so that no int64 index tensor of 2 G elements is ever made
+        out = torch.empty_like(idx)
+        for r in range(0, idx.shape[0], 2048):
+            out[r:r + 2048] = codes[idx[r:r + 2048].long()]
+        return out
+
+    a, b = fp8(ia), fp8(ib)
+    assert a.numel() > (1 << 31)
+    d = _gemm_nt(a, b, torch.float32, None)
+    bf = vals[ib.long()]
+    for r in (0, 8192, 16384, 24576, 32768 - 2048, 33024 - 2048):   # the last two blocks straddle / lie behind 2 GiB
+        ref = vals[ia[r:r + 2048].long()] @ bf.t()                     # exact: |sum| <= 4 * 65536 < 2^24
+        assert torch.equal(d[r:r + 2048], ref), r
