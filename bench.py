@@ -431,6 +431,32 @@ def quant_dual_kernel_ms(bufs, states, reps):
     return event_time_ms(fn, reps, warm=8)
 
 
+def stream_probe_ms(bufs, reps):
+    """The bandwidth yardsticks of the library (ntfp8_stream_probe: the flat quantise kernel's grid and access pattern
+    without its arithmetic and reduction) on the same rotating tensors: read-only, 2 bytes read per byte written (the
+    traffic of a bf16 -> fp8 cast), copy.  Milliseconds per launch."""
+    import torch
+
+    from nanotron_amd import _native as nt
+
+    dev = bufs[0].device
+    nbytes = bufs[0].numel() * bufs[0].element_size()
+    dst = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(2)]
+    st = nt.stream_ptr(dev)
+    res = {}
+    for name, mode in (("read_only", 0), ("read_2B_write_1B", 1), ("copy", 2)):
+        k = [0]
+
+        def fn():
+            i = k[0]
+            k[0] += 1
+            nt.check(nt.lib.ntfp8_stream_probe(mode, bufs[i % len(bufs)].data_ptr(), nbytes, dst[i % 2].data_ptr(), st),
+                     "ntfp8_stream_probe")
+
+        res[name] = event_time_ms(fn, reps, warm=8)
+    return res
+
+
 def quant_report(device, traffic):
     """The `quant` object of the JSON line: the fused quantise kernel on benchmark configuration 2 (bf16 [4096,4096],
     8 rotating buffers so that the input does not sit in the memory-side cache), the both-formats-in-one-pass kernel on
@@ -447,12 +473,18 @@ def quant_report(device, traffic):
     qb = 3.0 * 4096 * 4096
     q_avg = sum(qms.values()) / len(qms)
     dual_ms = quant_dual_kernel_ms(bufs, states, 64)
+    probe = stream_probe_ms(bufs, 64)
     rep = {"metric": "amax+quant GB/s", "value": round(qb / (q_avg * 1e-3) / 1e9, 1), "unit": "GB/s",
            "workload": "bf16 [4096,4096] fused amax+roll+scale+cast, 8 rotating buffers",
            "ms": {k: round(v, 5) for k, v in qms.items()},
            "roofline": {"bound": "hbm", "achieved": round(qb / (q_avg * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                         "frac": round(qb / (q_avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4), "traffic": traffic["quant"],
-                        "algorithmic_bytes": qb, "kernel": "quant_flat_kernel"},
+                        "algorithmic_bytes": qb, "kernel": "quant_flat_kernel",
+                        "frac_of_yardstick": round(probe["read_2B_write_1B"] / q_avg, 4)},
+           "yardstick": {"what": "ntfp8_stream_probe on the same tensors: same grid and 128-bit streaming accesses, no arithmetic, "
+                                 "no reduction",
+                         **{k: {"ms": round(v, 5), "GBps": round(b * 4096 * 4096 / (v * 1e-3) / 1e9, 1)}
+                            for (k, v), b in zip(probe.items(), (2.0, 3.0, 4.0))}},
            "both_formats_one_pass": {"ms": round(dual_ms, 5), "algorithmic_bytes": 4.0 * 4096 * 4096,
                                      "GBps": round(4.0 * 4096 * 4096 / (dual_ms * 1e-3) / 1e9, 1),
                                      "frac": round(4.0 * 4096 * 4096 / (dual_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
@@ -468,8 +500,12 @@ def quant_report(device, traffic):
         ms = quant_kernel_ms(lb, st, 32)
         avg = sum(ms.values()) / len(ms)
         nbytes = 3.0 * shape[0] * shape[1]
+        pr = stream_probe_ms(lb, 32)
         large[f"{shape[0]}x{shape[1]}"] = {"ms": round(avg, 5), "GBps": round(nbytes / (avg * 1e-3) / 1e9, 1),
-                                            "frac": round(nbytes / (avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)}
+                                            "frac": round(nbytes / (avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+                                            "yardstick_read_2B_write_1B_ms": round(pr["read_2B_write_1B"], 5),
+                                            "yardstick_read_only_GBps": round(2.0 * shape[0] * shape[1] / (pr["read_only"] * 1e-3) / 1e9, 1),
+                                            "frac_of_yardstick": round(pr["read_2B_write_1B"] / avg, 4)}
         del lb
     rep["large_tensors"] = large
     return rep
@@ -535,27 +571,158 @@ def probe(device):
 
 
 # ------------------------------------------------------------------------------------ vendor library, for comparison
-def workgroup_timeline(device):
-    """Where a workgroup of the GEMM kernel spends its time, read from the kernel itself: the profiling build of the
-    library (libntfp8_stamps.so, -DNTFP8_STAMPS) stamps the 100 MHz wall clock five times per workgroup and records
-    the CU it ran on.  Four launches without a half-tile tail: one round at K = 4096 and at K = 14336, three rounds, and
-    the seven-round dgrad + wgrad launch of the down projection."""
+def _profiling_lib(path):
+    """A profiling build of the library (nanotron_amd/profiling/, `python -m nanotron_amd.build --profiling`)."""
     import ctypes
 
-    import numpy as np
-    import torch
-
     from nanotron_amd import _native as nt
-    from nanotron_amd.fp8 import DTypes, FP8Tensor
 
-    path = os.path.join(ROOT, "nanotron_amd", "libntfp8_stamps.so")
     if not os.path.exists(path):
-        raise FileNotFoundError(f"{path}: build it with `python -m nanotron_amd.build`")
+        raise FileNotFoundError(f"{path}: build it with `python -m nanotron_amd.build --profiling`")
     lib = ctypes.CDLL(path)
     lib.ntfp8_gemm_batch.restype = ctypes.c_int
     lib.ntfp8_gemm_batch.argtypes = [ctypes.POINTER(nt.GemmDesc), ctypes.c_int, ctypes.c_void_p]
     lib.ntfp8_debug_stamps.restype = ctypes.c_int
     lib.ntfp8_debug_stamps.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+    lib.ntfp8_debug_set_tile_order.restype = ctypes.c_int
+    lib.ntfp8_debug_set_tile_order.argtypes = [ctypes.c_int]
+    return lib
+
+
+def _run_gemms(lib, probs, st):
+    """One ntfp8_gemm_batch call of `lib`; a problem is (a, b, out, b_transposed, a_transposed, d_dtype)."""
+    from nanotron_amd import _native as nt
+    from nanotron_amd.fp8 import DTypes
+
+    d = (nt.GemmDesc * len(probs))()
+    for e, (a, b, out, bt, at, dd) in zip(d, probs):
+        e.A, e.scale_a, e.B, e.scale_b, e.D = (a.data_ptr(), a.fp8_meta.scale.data_ptr(), b.data_ptr(),
+                                               b.fp8_meta.scale.data_ptr(), out.data_ptr())
+        (e.K, e.M) = a.shape if at else a.shape[::-1]
+        e.N = b.shape[1] if bt else b.shape[0]
+        e.fmt_a = 0 if a.fp8_meta.dtype == DTypes.FP8E4M3 else 1
+        e.fmt_b = 0 if b.fp8_meta.dtype == DTypes.FP8E4M3 else 1
+        e.d_dtype, e.accumulate, e.b_transposed, e.a_transposed = dd, 0, int(bt), int(at)
+    rc = lib.ntfp8_gemm_batch(d, len(probs), st)
+    assert rc == 0, rc
+
+
+def _pcts(v):
+    import numpy as np
+
+    return {k: round(float(np.percentile(v, p)), 2) for k, p in (("p10", 10), ("p50", 50), ("p90", 90), ("max", 100))}
+
+
+def _stamp_report(lib, n, k_tiles):
+    """Phases of the `n` workgroups of the last big-kernel launch of `lib`, from the stamps they left."""
+    import numpy as np
+
+    pcts = _pcts
+    buf = np.zeros(n * 8, dtype=np.uint64)
+    rc = lib.ntfp8_debug_stamps(buf.ctypes.data, buf.nbytes)
+    assert rc == 0, rc
+    s = buf.reshape(n, 8).astype(np.int64)
+    t = s[:, :5] * 0.01   # 100 MHz ticks -> us
+    t0, t_end = t[:, 0].min(), t[:, 4].max()
+    hw, xcc = s[:, 5] & 0xFFFFFFFF, (s[:, 5] >> 32) & 0xF
+    cycles = (s[:, 7] - s[:, 6]).astype(np.float64)   # shader-clock cycles of the K loop
+    cu = (xcc << 16) | (((hw >> 13) & 7) << 8) | (((hw >> 12) & 1) << 4) | ((hw >> 8) & 0xF)
+    ids = np.unique(cu)
+    handover, idle_end, per_cu = [], [], []
+    for c in ids:
+        idx = np.where(cu == c)[0]
+        idx = idx[np.argsort(t[idx, 0])]
+        per_cu.append(len(idx))
+        idle_end.append(t_end - t[idx[-1], 4])
+        handover += [t[b, 0] - t[a, 4] for a, b in zip(idx, idx[1:])]
+    loop = t[:, 2] - t[:, 1]
+    out = {"workgroups": n, "span_us": round(float(t_end - t0), 1), "cus": int(len(ids)),
+           "workgroups_per_cu": [int(min(per_cu)), int(max(per_cu))],
+           "us_per_workgroup": {"entry_to_first_tile": pcts(t[:, 1] - t[:, 0]), "k_loop": pcts(loop),
+                                "epilogue_issue": pcts(t[:, 3] - t[:, 2]), "store_drain": pcts(t[:, 4] - t[:, 3]),
+                                "whole": pcts(t[:, 4] - t[:, 0])},
+           "k_loop_cycles_per_k_tile_p50": round(float(np.median(cycles)) / k_tiles, 1),
+           "k_loop_us_per_k_tile_p50": round(float(np.median(loop)) / k_tiles, 3),
+           "k_loop_shader_clock_ghz_p50": round(float(np.median(cycles / (loop * 1e3))), 3),
+           "cu_idle_before_launch_end_us": pcts(idle_end),
+           "k_loop_p50_by_xcd_us": [round(float(np.median(loop[xcc == k])), 1) for k in range(8)],
+           "last_store_p50_by_xcd_us": [round(float(np.median([t[np.where(cu == c)[0], 4].max() - t0
+                                                               for c in ids if (c >> 16) == k])), 1) for k in range(8)]}
+    if handover:
+        out["handover_on_a_cu_us"] = pcts(handover)
+    return out
+
+
+def loop_experiments(device, reps=3, launches=24):
+    """What the K loop of a whole tile pays for, piece by piece, under sustained load: the experiment builds of the
+    profiling library (nanotron_amd/build.py: EXPERIMENTS; parts of the loop left out, or idle cycles put in) run the
+    one-round forward GEMMs of the O projection (K = 4096) and of the down projection (K = 14336) `launches` times
+    back to back on rotating operand sets, alternating between the builds.  Per build: microseconds per launch (HIP
+    events, best of `reps`), and from the stamps of the last launch the cycles per K-tile and the shader clock."""
+    import torch
+
+    from nanotron_amd import _native as nt
+    from nanotron_amd.build import EXPERIMENTS, experiment_lib
+    from nanotron_amd.fp8 import DTypes, FP8Tensor
+
+    libs = [(name, _profiling_lib(experiment_lib(name))) for name in EXPERIMENTS]
+    g = torch.Generator(device=device).manual_seed(5)
+    st = nt.stream_ptr(device)
+    bf16 = nt.TORCH_TO_NT[torch.bfloat16]
+    out = {}
+    for tag, K, nsets in (("o fwd 4096x4096x4096", 4096, 8), ("down fwd 4096x4096x14336", 14336, 4)):
+        sets = []
+        for _ in range(nsets):
+            x = FP8Tensor(torch.randn(TOKENS, K, generator=g, device=device).to(torch.bfloat16), DTypes.FP8E4M3)
+            w = FP8Tensor((torch.randn(4096, K, generator=g, device=device) * 0.02).to(torch.bfloat16), DTypes.FP8E4M3)
+            sets.append((x, w, torch.empty(TOKENS, 4096, dtype=torch.bfloat16, device=device)))
+        res = {name: {"us": []} for name, _ in libs}
+        vendor = "hipblaslt (vendor kernel, same operands, no stamps)"
+        res[vendor] = {"us": []}
+        one = torch.tensor(1.0, device=device)
+        views = [(x.as_subclass(torch.Tensor).view(torch.float8_e4m3fn), w.as_subclass(torch.Tensor).view(torch.float8_e4m3fn))
+                 for x, w, _ in sets]
+        for _ in range(reps):
+            kv = [0]
+
+            def vfn():
+                a, b = views[kv[0] % nsets]
+                kv[0] += 1
+                torch._scaled_mm(a, b.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+
+            res[vendor]["us"].append(round(event_time_ms(vfn, launches, warm=4) * 1e3, 1))
+            for name, lib in libs:
+                k = [0]
+
+                def fn():
+                    x, w, y = sets[k[0] % nsets]
+                    k[0] += 1
+                    _run_gemms(lib, [(x, w, y, False, False, bf16)], st)
+
+                res[name]["us"].append(round(event_time_ms(fn, launches, warm=4) * 1e3, 1))
+                rep = _stamp_report(lib, 256, K // 128)
+                res[name].update({"cycles_per_k_tile": rep["k_loop_cycles_per_k_tile_p50"],
+                                  "clock_ghz": rep["k_loop_shader_clock_ghz_p50"]})
+        for name in res:
+            res[name]["us_best"] = min(res[name]["us"])
+            res[name]["tflops"] = round(2.0 * TOKENS * 4096 * K / res[name]["us_best"] / 1e6, 1)
+        out[tag] = res
+        del sets
+    return out
+
+
+def workgroup_timeline(device):
+    """Where a workgroup of the GEMM kernel spends its time, read from the kernel itself: the profiling build of the
+    library (nanotron_amd/profiling/libntfp8_stamps.so, -DNTFP8_STAMPS) stamps the 100 MHz wall clock five times per
+    workgroup and records the CU it ran on.  Four launches without a half-tile tail: one round at K = 4096 and at
+    K = 14336, three rounds, and the seven-round dgrad + wgrad launch of the down projection."""
+    import torch
+
+    from nanotron_amd import _native as nt
+    from nanotron_amd.build import LIB_STAMPS
+    from nanotron_amd.fp8 import DTypes, FP8Tensor
+
+    lib = _profiling_lib(LIB_STAMPS)
     g = torch.Generator(device=device).manual_seed(1)
 
     def q(shape, std, dt):
@@ -564,55 +731,10 @@ def workgroup_timeline(device):
     st = nt.stream_ptr(device)
 
     def run(probs):
-        d = (nt.GemmDesc * len(probs))()
-        for e, (a, b, out, bt, at, dd) in zip(d, probs):
-            e.A, e.scale_a, e.B, e.scale_b, e.D = (a.data_ptr(), a.fp8_meta.scale.data_ptr(), b.data_ptr(),
-                                                   b.fp8_meta.scale.data_ptr(), out.data_ptr())
-            (e.K, e.M) = a.shape if at else a.shape[::-1]
-            e.N = b.shape[1] if bt else b.shape[0]
-            e.fmt_a = 0 if a.fp8_meta.dtype == DTypes.FP8E4M3 else 1
-            e.fmt_b = 0 if b.fp8_meta.dtype == DTypes.FP8E4M3 else 1
-            e.d_dtype, e.accumulate, e.b_transposed, e.a_transposed = dd, 0, int(bt), int(at)
-        rc = lib.ntfp8_gemm_batch(d, len(probs), st)
-        assert rc == 0, rc
-
-    def pcts(v):
-        return {k: round(float(np.percentile(v, p)), 2) for k, p in (("p10", 10), ("p50", 50), ("p90", 90), ("max", 100))}
+        _run_gemms(lib, probs, st)
 
     def report(n, k_tiles):
-        buf = np.zeros(n * 8, dtype=np.uint64)
-        rc = lib.ntfp8_debug_stamps(buf.ctypes.data, buf.nbytes)
-        assert rc == 0, rc
-        s = buf.reshape(n, 8).astype(np.int64)
-        t = s[:, :5] * 0.01   # 100 MHz ticks -> us
-        t0, t_end = t[:, 0].min(), t[:, 4].max()
-        hw, xcc = s[:, 5] & 0xFFFFFFFF, (s[:, 5] >> 32) & 0xF
-        cycles = (s[:, 7] - s[:, 6]).astype(np.float64)   # shader-clock cycles of the K loop
-        cu = (xcc << 16) | (((hw >> 13) & 7) << 8) | (((hw >> 12) & 1) << 4) | ((hw >> 8) & 0xF)
-        ids = np.unique(cu)
-        handover, idle_end, per_cu = [], [], []
-        for c in ids:
-            idx = np.where(cu == c)[0]
-            idx = idx[np.argsort(t[idx, 0])]
-            per_cu.append(len(idx))
-            idle_end.append(t_end - t[idx[-1], 4])
-            handover += [t[b, 0] - t[a, 4] for a, b in zip(idx, idx[1:])]
-        loop = t[:, 2] - t[:, 1]
-        out = {"workgroups": n, "span_us": round(float(t_end - t0), 1), "cus": int(len(ids)),
-               "workgroups_per_cu": [int(min(per_cu)), int(max(per_cu))],
-               "us_per_workgroup": {"entry_to_first_tile": pcts(t[:, 1] - t[:, 0]), "k_loop": pcts(loop),
-                                    "epilogue_issue": pcts(t[:, 3] - t[:, 2]), "store_drain": pcts(t[:, 4] - t[:, 3]),
-                                    "whole": pcts(t[:, 4] - t[:, 0])},
-               "k_loop_cycles_per_k_tile_p50": round(float(np.median(cycles)) / k_tiles, 1),
-               "k_loop_us_per_k_tile_p50": round(float(np.median(loop)) / k_tiles, 3),
-               "k_loop_shader_clock_ghz_p50": round(float(np.median(cycles / (loop * 1e3))), 3),
-               "cu_idle_before_launch_end_us": pcts(idle_end),
-               "k_loop_p50_by_xcd_us": [round(float(np.median(loop[xcc == k])), 1) for k in range(8)],
-               "last_store_p50_by_xcd_us": [round(float(np.median([t[np.where(cu == c)[0], 4].max() - t0
-                                                                   for c in ids if (c >> 16) == k])), 1) for k in range(8)]}
-        if handover:
-            out["handover_on_a_cu_us"] = pcts(handover)
-        return out
+        return _stamp_report(lib, n, k_tiles)
 
     T = TOKENS
     x, w = q((T, 4096), 1.0, DTypes.FP8E4M3), q((4096, 4096), 0.02, DTypes.FP8E4M3)
@@ -643,8 +765,6 @@ def workgroup_timeline(device):
         res[tag] = report(n, kt)
     # what the fetch traffic costs: the same launches with the XCD-aware tile order switched off (every XCD then pulls
     # every operand panel through its own L2)
-    lib.ntfp8_debug_set_tile_order.restype = ctypes.c_int
-    lib.ntfp8_debug_set_tile_order.argtypes = [ctypes.c_int]
     for tag, probs, n, kt in cases[1:3]:
         for plain in (1, 0):
             assert lib.ntfp8_debug_set_tile_order(plain) == 0
@@ -757,8 +877,8 @@ def main():
         probe(device)
         return
     if args.workload == "wg-timeline":
-        print(json.dumps({"workload": "per-workgroup wall-clock stamps inside gemm_nt_big_kernel (profiling build)",
-                          "launches": workgroup_timeline(device)}))
+        print(json.dumps({"workload": "per-workgroup wall-clock stamps inside gemm_nt_big_kernel (profiling builds)",
+                          "launches": workgroup_timeline(device), "k_loop_experiments": loop_experiments(device)}))
         return
     if args.workload == "vendor-gemm":
         n = args.operand_sets
@@ -824,7 +944,9 @@ def main():
             "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(achieved / PEAK_FP8_TFLOPS, 4),
                          "traffic": traffic["gemm"],
-                         "traffic_unit": "bytes per step, all GEMM launches (fetch + write counters)",
+                         "traffic_unit": "bytes per step over all GEMM launches: fills of the eight XCD L2s (FETCH_SIZE) + writes "
+                                         "(WRITE_SIZE); L2-fill traffic, not HBM bytes (re-fetched panels can come from the "
+                                         "256 MB memory-side cache)",
                          "traffic_source": traffic["source"],
                          "algorithmic_bytes": gemm_algorithmic_bytes(),
                          "kernel": "gemm_nt_big_kernel", "timing": "HIP events around every GEMM call inside the step",

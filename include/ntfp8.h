@@ -237,6 +237,17 @@ int ntfp8_gemm_batch(const ntfp8_gemm_desc* problems, int count, void* stream);
 int ntfp8_amax_finalize(void* workspace, int fmt, int margin, float* scale_state, float* amax_history,
                         int history_len, float* amax_out, float* scale_used_out, void* stream);
 
+/* Bandwidth yardstick: a kernel with the access pattern of the flat quantise kernels (same workgroup size, same grid,
+ * 128-bit streaming loads and stores) and none of their arithmetic, so that a quantise figure can be set against what
+ * the memory system gives that pattern on the same GPU in the same run.  It has no counterpart in the reference; it is
+ * a measurement aid for the benchmark.  `bytes` (a multiple of 32) are read from src (16-byte aligned);
+ * NTFP8_PROBE_READ writes nothing (dst: 16 bytes that are left alone in practice), NTFP8_PROBE_HALF writes bytes / 2
+ * to dst (the traffic of a 16-bit -> fp8 cast), NTFP8_PROBE_COPY writes bytes. */
+#define NTFP8_PROBE_READ 0
+#define NTFP8_PROBE_HALF 1
+#define NTFP8_PROBE_COPY 2
+int ntfp8_stream_probe(int mode, const void* src, int64_t bytes, void* dst, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

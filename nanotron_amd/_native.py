@@ -70,6 +70,7 @@ SIGNATURES = {
     "ntfp8_gemm": (_i, [_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i64, _i64, _i64, _i, _vp]),
     "ntfp8_gemm_batch": (_i, [_c.POINTER(GemmDesc), _i, _vp]),
     "ntfp8_amax_finalize": (_i, [_vp, _i, _i, _vp, _vp, _i, _vp, _vp, _vp]),
+    "ntfp8_stream_probe": (_i, [_i, _vp, _i64, _vp, _vp]),
 }
 
 for _name, (_res, _args) in SIGNATURES.items():

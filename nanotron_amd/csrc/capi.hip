@@ -16,6 +16,7 @@ int run_transpose(const void* in, int64_t rows, int64_t cols, void* out, hipStre
 int run_update_scale(const float* amax, const float* old_scale, int fmt, int margin, float* out, int64_t n,
                      hipStream_t st);
 int run_amax_finalize(Workspace* ws, const ScalarIO& io, hipStream_t st);
+int run_stream_probe(int mode, const void* src, int64_t bytes, void* dst, hipStream_t st);
 int run_quant_delayed_batch(const QuantDesc* q, int count, hipStream_t st);
 int run_gemm(const GemmDesc& g, hipStream_t st);
 int run_gemm_batch(const GemmDesc* g, int n, hipStream_t st);
@@ -392,6 +393,16 @@ int ntfp8_amax_finalize(void* workspace, int fmt, int margin, float* scale_state
         return NTFP8_ERR_ALIGN;
     ScalarIO io = {nullptr, amax_out, scale_used_out, scale_state, amax_history, history_len, fmt, margin};
     return run_amax_finalize(static_cast<Workspace*>(workspace), io, static_cast<hipStream_t>(stream));
+}
+
+int ntfp8_stream_probe(int mode, const void* src, int64_t bytes, void* dst, void* stream) {
+    if (!src || !dst) return NTFP8_ERR_NULL;
+    if (mode < NTFP8_PROBE_READ || mode > NTFP8_PROBE_COPY) return NTFP8_ERR_ENUM;
+    if (bytes < 32 || bytes % 32 != 0 || bytes > (1LL << 46)) return NTFP8_ERR_SIZE;
+    if (!is_aligned(src, 16) || !is_aligned(dst, 16)) return NTFP8_ERR_ALIGN;
+    const size_t written = mode == NTFP8_PROBE_READ ? 16 : (mode == NTFP8_PROBE_HALF ? (size_t)bytes / 2 : (size_t)bytes);
+    if (overlap(src, (size_t)bytes, dst, written)) return NTFP8_ERR_ALIAS;
+    return run_stream_probe(mode, src, bytes, dst, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -91,8 +91,16 @@ __host__ __device__ inline float update_scale(float amax, float old_scale, int f
     if ((ab >> 31) || mag == 0u) return old_scale;   // amax <= 0: scale held
     const float ratio = fp8_max_of(fmt) / amax;      // IEEE round-to-nearest division
     if ((f32_bits(ratio) & 0x7fffffffu) >= kInfBits) return bits_f32(kInfBits);
-    const float l2 = (float)log2((double)ratio);
-    const int e = (int)floorf(l2) - margin;
+    // floor(float(log2(ratio))).  Rounded to float, the logarithm reaches the next integer only for a ratio within a few
+    // tens of mantissa steps below a power of two (the spacing of floats near |k| <= 128 is at most 44 steps of
+    // d log2 / d mantissa = 8.6e-8): every other normal ratio gives its own exponent, read off the bits.  The double
+    // logarithm, a long software routine that the last workgroup of a quantise launch runs on one lane while the
+    // whole GPU waits for it, is only evaluated for those few and for subnormal ratios.
+    const uint32_t rb = f32_bits(ratio);
+    int fl;
+    if ((rb >> 23) != 0u && (rb & 0x7fffffu) < 0x7fff00u) fl = (int)(rb >> 23) - 127;
+    else fl = (int)floorf((float)log2((double)ratio));
+    const int e = fl - margin;
     const int ae = e < 0 ? -e : e;
     if (ae >= 128) return e < 0 ? 0.0f : bits_f32(kInfBits);
     // 2^e as a bit pattern (normal for e >= -126, subnormal below)

@@ -38,10 +38,25 @@ __device__ unsigned long long g_stamps[kStampSlots * 8];
 __device__ int g_plain_tile_order = 0;
 #define NTFP8_STAMP(var) var = wall_clock64()
 #define NTFP8_CYCLES(var) var = __builtin_readcyclecounter()
+// Timing experiments on the K loop of whole tiles, chosen when a profiling build is compiled (the results of such a
+// build are wrong, only its stamps mean something).  -DNTFP8_KNOCKOUT=<bits> leaves parts of the loop out: 1 the global
+// loads (stale registers are deposited), 2 the deposits into LDS, 4 the workgroup barrier, 8 the LDS reads of the B
+// fragments, 16 those of the A fragments.  -DNTFP8_IDLE=<n> lets every wave sleep 64 n cycles behind the barrier of
+// every K-tile.
+#ifndef NTFP8_KNOCKOUT
+#define NTFP8_KNOCKOUT 0
+#endif
+#ifndef NTFP8_IDLE
+#define NTFP8_IDLE 0
+#endif
+constexpr int kKnockout = NTFP8_KNOCKOUT, kIdle = NTFP8_IDLE;
 #else
 #define NTFP8_STAMP(var) (void)0
 #define NTFP8_CYCLES(var) (void)0
+constexpr int kKnockout = 0, kIdle = 0;
 #endif
+constexpr bool kNoLoads = kKnockout & 1, kNoDeposits = kKnockout & 2, kNoBarrier = kKnockout & 4, kNoBReads = kKnockout & 8,
+               kNoAReads = kKnockout & 16;
 
 
 constexpr int kBigN = 256;
@@ -556,7 +571,7 @@ void gemm_nt_big_kernel(const BigLaunch L) {
             for (int i = 0; i < MI; ++i) {
                 // fa[i] is dead after its two MFMAs; it is refilled with the fragment of the next tile one step later
                 acc[i][6] = mfma_16x16x128<FA, FB>(frag(fb[2]), frag(fa[i]), acc[i][6]);
-                if (prefetch && i > 0) {
+                if (prefetch && !kNoAReads && i > 0) {
                     fa[i - 1][0] = rd_a(s1, i - 1, 0);
                     fa[i - 1][1] = rd_a(s1, i - 1, 1);
                 }
@@ -566,10 +581,10 @@ void gemm_nt_big_kernel(const BigLaunch L) {
 #pragma unroll
                     for (int l = i * kBackLoads / MI; l < (i + 1) * kBackLoads / MI; ++l) issue(kt + NS, l);
                 }
-                if (prefetch && i < 4) fb[i >> 1][i & 1] = rd_b(s1, i >> 1, i & 1);
+                if (prefetch && !kNoBReads && i < 4) fb[i >> 1][i & 1] = rd_b(s1, i >> 1, i & 1);
                 sched_fence();
             }
-            if constexpr (prefetch) {
+            if constexpr (prefetch && !kNoAReads) {
                 fa[MI - 1][0] = rd_a(s1, MI - 1, 0);
                 fa[MI - 1][1] = rd_a(s1, MI - 1, 1);
             }
@@ -588,10 +603,15 @@ void gemm_nt_big_kernel(const BigLaunch L) {
             // than from the memory-side cache stalled the barrier.
             v4i g[NL];
             const int wr_lane = wave * 1024 + lane * 16;   // a wave-level load covers 1 KB of a stage: 16 bytes per lane
+            if constexpr (kNoLoads) {
+#pragma unroll
+                for (int l = 0; l < NL; ++l) g[l] = (v4i){l, lane, 0, 0};
+            }
             auto request = [&](int ktile, int l) {
-                g[l] = l < LA ? reg_load16(ra, a_off[l], ktile * a_step) : reg_load16(rb, b_off[l - LA], ktile * b_step);
+                if constexpr (!kNoLoads) g[l] = l < LA ? reg_load16(ra, a_off[l], ktile * a_step) : reg_load16(rb, b_off[l - LA], ktile * b_step);
             };
             auto deposit = [&](int s, int l) {
+                if constexpr (kNoDeposits) return;
                 if (l < LA) *reinterpret_cast<v4i*>(&sA[s][wr_lane + l * (kBigWaves * 1024)]) = g[l];
                 else *reinterpret_cast<v4i*>(&sB[s][wr_lane + (l - LA) * (kBigWaves * 1024)]) = g[l];
             };
@@ -608,8 +628,8 @@ void gemm_nt_big_kernel(const BigLaunch L) {
 #pragma unroll
                     for (int i = 0; i < MI; ++i) {
                         acc[i][j] = mfma_16x16x128<FA, FB>(frag(fb[j & 3]), frag(fa[i]), acc[i][j]);
-                        if (i == 0) fb[(j + 2) & 3][0] = rd_b(s, j + 2, 0);
-                        else if (i == 2) fb[(j + 2) & 3][1] = rd_b(s, j + 2, 1);
+                        if (i == 0) { if constexpr (!kNoBReads) fb[(j + 2) & 3][0] = rd_b(s, j + 2, 0); }
+                        else if (i == 2) { if constexpr (!kNoBReads) fb[(j + 2) & 3][1] = rd_b(s, j + 2, 1); }
                         else if (l < NL) {
                             const bool second = i == 3 || i == 5 || i == 7;   // slots 1,3 / 4,5 / 6,7 form the pairs
                             if (!second) { if (W) deposit(s ^ 1, l); }
@@ -625,7 +645,8 @@ void gemm_nt_big_kernel(const BigLaunch L) {
                     // the first front publishes tile 1, which the prologue sent straight to LDS: its loads are
                     // older than the NL requests of tile 2 queued above
                     if constexpr (!W) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(L ? NL : 0) : "memory");
-                    wg_barrier();
+                    if constexpr (!kNoBarrier) wg_barrier();
+                    if constexpr (kIdle > 0) __builtin_amdgcn_s_sleep(kIdle);
                 }
             };
             // prologue: tiles 0 and 1 straight into LDS

@@ -74,10 +74,6 @@ __device__ __forceinline__ void wg_barrier() {
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
 }
-__device__ __forceinline__ void mfma_priority(bool high) {
-    if (high) __builtin_amdgcn_s_setprio(1);
-    else __builtin_amdgcn_s_setprio(0);
-}
 // x of lanes 32..63 <-> y of lanes 0..31 (V_PERMLANE32_SWAP)
 __device__ __forceinline__ void swap_halves(uint32_t& x, uint32_t& y) {
     typedef unsigned v2u __attribute__((ext_vector_type(2)));

@@ -145,7 +145,7 @@ __device__ __forceinline__ uint8_t encode1(float x, float scale) {
 // force.  It takes one round trip out of the dependent chain at the end of the kernel.
 struct EpiloguePrefetch {
     float hist_prev;  // hist[lane - 1] (lanes 1 .. hist_len-1; histories of up to 64 entries)
-    float scale;      // *scale_state
+    float scale;      // *scale_state; amax-only mode: *old_scale (1.0 if there is none)
 };
 __device__ __forceinline__ EpiloguePrefetch prefetch_epilogue(const ScalarIO& io, int mode) {
     EpiloguePrefetch p = {0.0f, 1.0f};
@@ -153,6 +153,7 @@ __device__ __forceinline__ EpiloguePrefetch prefetch_epilogue(const ScalarIO& io
         const int lane = threadIdx.x;
         if (io.hist && io.hist_len <= 64 && lane >= 1 && lane < io.hist_len) p.hist_prev = io.hist[lane - 1];
         if (mode != kModeAmaxOnly) p.scale = *io.scale_state;
+        else if (io.old_scale) p.scale = *io.old_scale;
     }
     return p;
 }
@@ -177,8 +178,7 @@ __device__ inline void bookkeep(uint32_t bits, const ScalarIO& io, int mode, con
     const float a = __uint_as_float(bits);
     float used;
     if (mode == kModeAmaxOnly) {
-        const float old = io.old_scale ? *io.old_scale : 1.0f;
-        used = update_scale(a, old, io.fmt, io.margin);
+        used = update_scale(a, pre.scale, io.fmt, io.margin);
     } else {
         used = pre.scale;
     }
@@ -556,6 +556,37 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
         if (c0 + c < cols && r0 + tx < rows) out[(c0 + c) * rows + r0 + tx] = tile[tx][c];
 }
 
+// ---------------------------------------------------------------------------------------------
+// Bandwidth yardsticks: the access pattern of the flat quantise kernel (one 1024-thread workgroup per CU, two
+// 16-element groups per lane and trip, 128-bit non-temporal accesses) with the arithmetic and the reduction taken
+// out.  kProbeRead: 32 bytes read per group, nothing written.  kProbeHalf: 32 bytes read, 16 written (the traffic of
+// a bf16 -> fp8 cast).  kProbeCopy: 32 read, 32 written.
+enum ProbeMode { kProbeRead = NTFP8_PROBE_READ, kProbeHalf = NTFP8_PROBE_HALF, kProbeCopy = NTFP8_PROBE_COPY };
+template <int MODE>
+__global__ __launch_bounds__(kFlatThreads) void stream_probe_kernel(const u4* __restrict__ src, int64_t n_vec, u4* __restrict__ dst) {
+    const int64_t stride = (int64_t)gridDim.x * kFlatThreads;
+    int64_t i = (int64_t)blockIdx.x * kFlatThreads + threadIdx.x;
+    u4 seen = {0u, 0u, 0u, 0u};
+    auto one = [&](int64_t k) {
+        const u4 a = __builtin_nontemporal_load(src + 2 * k), b = __builtin_nontemporal_load(src + 2 * k + 1);
+        if constexpr (MODE == kProbeRead) seen = seen | (a ^ b);
+        else if constexpr (MODE == kProbeHalf) __builtin_nontemporal_store(a ^ b, dst + k);
+        else {
+            __builtin_nontemporal_store(a, dst + 2 * k);
+            __builtin_nontemporal_store(b, dst + 2 * k + 1);
+        }
+    };
+    for (; i + stride < n_vec; i += 2 * stride) {
+        one(i);
+        one(i + stride);
+    }
+    if (i < n_vec) one(i);
+    if constexpr (MODE == kProbeRead) {
+        // keeps the loads alive; a word of dst is written only if every bit of some lane's xor came out set
+        if ((seen.x & seen.y & seen.z & seen.w) == 0xffffffffu) reinterpret_cast<uint32_t*>(dst)[0] = 1u;
+    }
+}
+
 __global__ void update_scale_kernel(const float* amax, const float* old_scale, int fmt, int margin, float* out,
                                     int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -819,6 +850,18 @@ int run_transpose(const void* in, int64_t rows, int64_t cols, void* out, hipStre
     if (tiles > 0x7fffffff) return NTFP8_ERR_SIZE;
     hipLaunchKernelGGL(transpose_kernel, dim3((int)tiles), dim3(kThreads), 0, st, static_cast<const uint8_t*>(in), rows,
                        cols, static_cast<uint8_t*>(out));
+    return check_launch();
+}
+
+int run_stream_probe(int mode, const void* src, int64_t bytes, void* dst, hipStream_t st) {
+    clear_stale_error();
+    const int64_t n_vec = bytes / 32;
+    const int grid = grid_for((n_vec + 1) / 2, kFlatThreads, 1);
+    const u4* s = static_cast<const u4*>(src);
+    u4* d = static_cast<u4*>(dst);
+    if (mode == kProbeRead) hipLaunchKernelGGL((stream_probe_kernel<kProbeRead>), dim3(grid), dim3(kFlatThreads), 0, st, s, n_vec, d);
+    else if (mode == kProbeHalf) hipLaunchKernelGGL((stream_probe_kernel<kProbeHalf>), dim3(grid), dim3(kFlatThreads), 0, st, s, n_vec, d);
+    else hipLaunchKernelGGL((stream_probe_kernel<kProbeCopy>), dim3(grid), dim3(kFlatThreads), 0, st, s, n_vec, d);
     return check_launch();
 }
 
