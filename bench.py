@@ -73,9 +73,30 @@ def parse():
     p.add_argument("--fp8-activations", action="store_true",
                    help="every linear returns its output as an e4m3 FP8Tensor quantised in the GEMM epilogue "
                         "(no bf16 activation is written); not the headline configuration")
+    p.add_argument("--no-graph", action="store_true",
+                   help="linear workload: launch every step from Python instead of replaying HIP graphs of the steps "
+                        "(one graph per input set, captured after the correctness gate)")
     p.add_argument("--no-verify", action="store_true",
                    help="skip the correctness gate (profiling runs only: the line then says verified = false)")
     return p.parse_args()
+
+
+def capture_steps(mods, sets, wstream, fp8_out):
+    """One HIP graph per input set: the step is captured as the eager code issues it (same kernels, same order), the
+    graphs share one memory pool and are replayed in capture order, round robin.  The scaling state lives outside the
+    pool and carries over from replay to replay exactly as from eager step to eager step.  Every role must hold a scale
+    already (a role's first quantisation reads its amax on the host)."""
+    import torch
+
+    assert all(st.initialised for lin in mods for st in lin.scaling.values()), "run two eager steps before capturing"
+    graphs, pool = [], None
+    for j in range(len(sets)):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, pool=pool):
+            linear_step(mods, sets, j, wstream, fp8_out=fp8_out)
+        pool = g.pool()
+        graphs.append(g)
+    return graphs
 
 
 def flags_of(args):
@@ -157,6 +178,7 @@ def build_linears(device, nsets, fp8_out=False):
             if s_ < 2:   # what the correctness gate compares with
                 per_step.append((x, w, gy))
         lin.weight = sets[0]["w"][i]
+        lin.keep_quantised_grad = True   # the correctness gate compares the e5m2 bytes of dY too (switched off after it)
         mods.append(lin)
         cpu.append(per_step)
     return mods, sets, cpu
@@ -198,10 +220,12 @@ def verify_steps(mods, sets, cpu, wstream):
         def check(i, lin, x, y, saved):
             xc, wc, gc = cpu[i][step]
             errs = C.check_layer(f"step {step} {LINEARS[i][0]}", lin, refs[i], xc, wc, gc, y.detach(), x.grad,
-                                 lin.weight.main_grad, saved, step, i)
+                                 lin.weight.main_grad, saved, step, i, gq_gpu=lin.quantised_grad_output)
             for k, v in errs.items():
                 worst[k] = max(worst[k], v)
         linear_step(mods, sets, step, wstream, check=check)
+    for lin in mods:
+        lin.keep_quantised_grad, lin.quantised_grad_output = False, None
     return {k: float(f"{v:.3e}") for k, v in worst.items()}
 
 
@@ -893,7 +917,8 @@ def main():
         nsets = max(2, min(10, args.warmup + 2 * args.steps))
         mods, sets, cpu = build_linears(device, nsets, fp8_out=args.fp8_activations)
         wstream = torch.cuda.Stream(device=device) if args.weight_stream else None
-        step = lambda i: linear_step(mods, sets, i, wstream, fp8_out=args.fp8_activations)
+        eager_step = lambda i: linear_step(mods, sets, i, wstream, fp8_out=args.fp8_activations)
+        step = eager_step
         flops_step = sum(6.0 * TOKENS * N * K for _, K, N in LINEARS)
         first = 0
         if not args.no_verify and not args.fp8_activations:
@@ -905,6 +930,18 @@ def main():
                 sys.exit(1)
             first = 2
         del cpu
+        graph_note = None
+        if not args.no_graph and not args.weight_stream:
+            # two eager steps (the gate's, or these) have given every scaling role its first scale
+            for i in range(first, 2):
+                eager_step(i)
+            first = max(first, 2)
+            try:
+                graphs = capture_steps(mods, sets, wstream, args.fp8_activations)
+                step = lambda i: graphs[i % len(graphs)].replay()
+            except Exception as e:   # reported, not hidden: the line then says the steps were launched eagerly
+                graph_note = f"graph capture failed, eager launches instead: {type(e).__name__}: {e}"
+                torch.cuda.synchronize()
     else:
         bufs, states = build_quant(device)
         step = lambda i: quant_step(bufs, states, i)
@@ -929,7 +966,22 @@ def main():
     }
     if args.workload == "linear":
         value = flops_step / (ms_per_step * 1e-3) / 1e12
-        gf, gms, per_call = gemm_in_step_timing(step, first + args.warmup + args.steps, args.steps)
+        launch = "eager" if step is eager_step else "hip graph replay"
+        eager = None
+        if step is not eager_step:
+            # the same steps launched from Python, for comparison (and the passes the GEMM timing instruments)
+            for i in range(2):
+                eager_step(first + i)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for i in range(args.steps):
+                eager_step(first + 2 + i)
+            e_host = (time.perf_counter() - t1) / args.steps * 1e3
+            torch.cuda.synchronize()
+            e_ms = (time.perf_counter() - t1) / args.steps * 1e3
+            eager = {"ms_per_step": round(e_ms, 4), "host_ms_per_step": round(e_host, 4),
+                     "value": round(flops_step / (e_ms * 1e-3) / 1e12, 2)}
+        gf, gms, per_call = gemm_in_step_timing(eager_step, first + args.warmup + args.steps, args.steps)
         achieved = gf / (gms * 1e-3) / 1e12
         acts = "e4m3 activations out of the GEMM epilogue" if args.fp8_activations else "bf16 activations"
         out.update({
@@ -937,6 +989,7 @@ def main():
             "config": {"workload": f"llama3-8b decoder-block linears fwd+bwd, 4096 tokens, {acts}, bf16 master weights, "
                                    "delayed scaling hist 16, fresh seeded X/dY and perturbed weights every step",
                        "weight_requantisation": "second stream, per layer" if args.weight_stream else "compute stream, one batched call per step",
+                       "launch": launch, "launch_note": graph_note, "eager_launches": eager,
                        "tokens": TOKENS, "linears": [f"{n}:{k}->{o}" for n, k, o in LINEARS], "input_sets": len(sets),
                        "flags": flags_of(args), "flops_per_step": flops_step, "pct_fp8_peak": round(100 * value / PEAK_FP8_TFLOPS, 2)},
             "verified": ({"against": "CPU oracle, steps 0 and 1: amax / scales / histories / fp8 bytes bit-exact, "

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define NTFP8_VERSION 2
+#define NTFP8_VERSION 3
 #define NTFP8_WORKSPACE_BYTES 2048
 
 /* FP8 storage formats.  Reference: DTypes.FP8E4M3 / DTypes.FP8E5M2 (src/nanotron/fp8/dtypes.py:4-7),
@@ -96,6 +96,20 @@ int ntfp8_quantize_current(const void* x, int x_dtype, int64_t rows, int64_t col
                            float* amax_out, float* scale_used_out, void* out, void* out_t,
                            float* amax_history, int history_len, float* scale_state,
                            void* workspace, void* stream);
+
+/* The quantisation of a delayed-scaling role that may or may not hold a scale yet, decided on the device (the host
+ * reads nothing back, so the call can be captured in a HIP graph from a role's very first step): *initialised is a
+ * flag in device memory, 0.0 until a finite positive amax has been recorded.
+ *   *initialised == 0:  the result of ntfp8_quantize_current with the history arguments (the reference's scaling,
+ *                       src/nanotron/fp8/tensor.py:25-28: the scale comes from this tensor's own amax);
+ *   *initialised != 0:  the result of ntfp8_quantize_delayed, bit for bit (cast with *scale_state, history rolled,
+ *                       next scale stored), from two launches instead of one (amax pass, then cast: 5 bytes per 16-bit
+ *                       element instead of 3);
+ * and *initialised becomes 1.0 if this tensor's amax is finite and positive.  A caller that knows the role holds a scale
+ * calls ntfp8_quantize_delayed. */
+int ntfp8_quantize_first_use(const void* x, int x_dtype, int64_t rows, int64_t cols, int fmt, int margin, float* scale_state,
+                             float* amax_history, int history_len, float* initialised, float* amax_out,
+                             float* scale_used_out, void* out, void* out_t, void* workspace, void* stream);
 
 /* One delayed-scaling step in a single pass over x (no counterpart in the reference, which
  * has no amax history; semantics fixed by the benchmark configs: history 16, margin 0):

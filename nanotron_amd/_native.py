@@ -58,6 +58,7 @@ SIGNATURES = {
     "ntfp8_update_scaling_factor_host": (_f, [_f, _f, _i, _i]),
     "ntfp8_cast_to_fp8": (_i, [_vp, _i, _i64, _i64, _vp, _i, _vp, _vp, _vp]),
     "ntfp8_quantize_current": (_i, [_vp, _i, _i64, _i64, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp]),
+    "ntfp8_quantize_first_use": (_i, [_vp, _i, _i64, _i64, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "ntfp8_quantize_delayed": (_i, [_vp, _i, _i64, _i64, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "ntfp8_quantize_delayed_batch": (_i, [_c.POINTER(QuantDesc), _i, _vp]),
     "ntfp8_quantize_delayed_batch_static": (_i, [_c.POINTER(QuantDesc), _i, _vp]),

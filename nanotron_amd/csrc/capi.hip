@@ -194,6 +194,33 @@ int ntfp8_quantize_current(const void* x, int x_dtype, int64_t rows, int64_t col
                      scale_used_out, nullptr, none, st);
 }
 
+int ntfp8_quantize_first_use(const void* x, int x_dtype, int64_t rows, int64_t cols, int fmt, int margin, float* scale_state,
+                             float* amax_history, int history_len, float* initialised, float* amax_out,
+                             float* scale_used_out, void* out, void* out_t, void* workspace, void* stream) {
+    int64_t n;
+    if (!scale_state || !amax_history || !initialised || !amax_out || !scale_used_out || !workspace || (!out && !out_t))
+        return NTFP8_ERR_NULL;
+    int rc = check_quant_common(x, x_dtype, rows, cols, fmt, margin, &n);
+    if (rc) return rc;
+    if (history_len < 1 || history_len > kMaxHistory) return NTFP8_ERR_SIZE;
+    if (!is_aligned(scale_state, 4) || !is_aligned(amax_history, 4) || !is_aligned(initialised, 4) || !is_aligned(amax_out, 4) ||
+        !is_aligned(scale_used_out, 4) || !is_aligned(workspace, 4))
+        return NTFP8_ERR_ALIGN;
+    rc = check_outputs(x, x_dtype, n, out, out_t);
+    if (rc) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // launch 1: amax, the decision between this tensor's scale and the held one, history roll, next scale
+    ScalarIO io = {nullptr, amax_out, scale_used_out, scale_state, amax_history, history_len, fmt, margin, nullptr, nullptr,
+                   initialised};
+    rc = run_quant(kModeAmaxOnly, x, x_dtype, n, 1, fmt, nullptr, nullptr, nullptr, static_cast<Workspace*>(workspace), io,
+                   st);
+    if (rc) return rc;
+    // launch 2: the cast with the scale launch 1 chose
+    ScalarIO none = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, fmt, 0};
+    return run_quant(kModeCastOnly, x, x_dtype, rows, cols, fmt, static_cast<uint8_t*>(out), static_cast<uint8_t*>(out_t),
+                     scale_used_out, nullptr, none, st);
+}
+
 int ntfp8_quantize_delayed(const void* x, int x_dtype, int64_t rows, int64_t cols, int fmt, int margin,
                            float* scale_state, float* amax_history, int history_len, float* amax_out,
                            float* scale_used_out, void* out, void* out_t, void* workspace, void* stream) {

@@ -48,6 +48,9 @@ struct ScalarIO {
     // Transformer-Engine-shaped cast (tex.cast_to_fp8 takes `amax` and `scale_inv` tensors and updates both):
     const float* amax_in;    // not NULL: *amax_out = max(*amax_in, amax of this tensor), NaN from either side kept
     float* scale_inv_out;    // not NULL: receives 1 / (scale the bytes were produced with)
+    // First use of a delayed-scaling role (amax-only mode): 0.0 = no usable amax recorded yet, scale from this tensor's
+    // amax; anything else = the role holds a scale, *scale_state is used.  Set to 1.0 when this amax is finite and > 0.
+    float* init_flag;
 };
 
 // one tensor of a batched quantise call as the launchers see it (validated by the C entry point)

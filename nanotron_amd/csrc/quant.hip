@@ -178,7 +178,9 @@ __device__ inline void bookkeep(uint32_t bits, const ScalarIO& io, int mode, con
     const float a = __uint_as_float(bits);
     float used;
     if (mode == kModeAmaxOnly) {
-        used = update_scale(a, pre.scale, io.fmt, io.margin);
+        // (the flag and the held scale are read here, before lane 0 writes either below)
+        if (io.init_flag && *io.init_flag != 0.0f) used = *io.scale_state;
+        else used = update_scale(a, pre.scale, io.fmt, io.margin);
     } else {
         used = pre.scale;
     }
@@ -215,6 +217,7 @@ __device__ inline void bookkeep(uint32_t bits, const ScalarIO& io, int mode, con
         if (io.scale_out) *io.scale_out = used;
         if (io.scale_inv_out) *io.scale_inv_out = 1.0f / used;
         if (io.hist) *io.scale_state = update_scale(__uint_as_float(hm), used, io.fmt, io.margin);
+        if (io.init_flag && bits != 0u && bits < kInfBits) *io.init_flag = 1.0f;
     }
 }
 

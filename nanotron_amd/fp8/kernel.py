@@ -61,7 +61,7 @@ def _gemm_nt_fp8(a: FP8Tensor, b: FP8Tensor, dtype: DTypes, state: Optional[Dela
     from nanotron_amd.fp8.meta import FP8Meta
 
     assert dtype in _OUT_FMT, f"{dtype} is not an FP8 format"
-    if state is None or not state.initialised:
+    if state is None or not state.known_initialised:
         hp = (_gemm_nt_batch([(a, b, torch.float32, None, True, None, at)])[0] if bt
               else _gemm_nt(a, b, torch.float32, None, bias))
         return FP8Tensor(hp, dtype, state=state, with_transpose=with_transpose)

@@ -47,6 +47,11 @@ class FP8Linear(nn.Linear):
         self.out_dtype = out_dtype
         self.fp8_output_transpose = fp8_output_transpose
         self.accumulate_grad = accumulate_grad
+        # True: every backward leaves the quantised output gradient (the FP8Tensor both backward GEMMs read) in
+        # `self.quantised_grad_output`, as autograd keeps the quantised input in `saved_tensors`; off by default, the
+        # reference drops it (linear.py:102) and it would pin the bytes until the next backward
+        self.keep_quantised_grad = False
+        self.quantised_grad_output = None
         self.scaling = None
         self._weight_ready = None
         if self.weight.device != torch.device("cpu"):
@@ -274,6 +279,8 @@ class _FP8Matmul(torch.autograd.Function):
                 x_plain and a_transposed_supported(g2d.shape[1], input.shape[1], g2d.shape[0]))
             grad_output = FP8Tensor(g2d, dtype=DTypes.FP8E5M2, state=scaling["output_grad"] if scaling else None,
                                     with_transpose=with_t)
+            if module is not None and module.keep_quantised_grad:
+                module.quantised_grad_output = grad_output   # for checkers: the e5m2 operand of dgrad and wgrad
 
         wants_dx = ctx.needs_input_grad[0] or (ctx.has_handle and ctx.needs_input_grad[6])
         grad_input = None

@@ -35,7 +35,7 @@ def requantize_fp8_weights(module_or_modules, stream: Optional[torch.cuda.Stream
     rest = layers
     if stream is None:
         # weights whose delayed-scaling role already holds a scale go through one batched library call per device
-        ready = [lin for lin in layers if lin.scaling is not None and lin.scaling["weight"].initialised]
+        ready = [lin for lin in layers if lin.scaling is not None and lin.scaling["weight"].known_initialised]
         by_device = {}
         for lin in ready:
             by_device.setdefault(lin.weight.device, []).append(lin)

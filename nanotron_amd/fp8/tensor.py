@@ -36,7 +36,12 @@ class DelayedScaling:
 
     The first quantisation through a fresh state (no finite positive amax recorded yet) uses
     current scaling, exactly the reference's behaviour; from then on every step is a single
-    fused pass: cast with the held scale, amax, history roll, next scale."""
+    fused pass: cast with the held scale, amax, history roll, next scale.
+
+    Whether a usable amax has been recorded is a flag in device memory, and the kernels of a role's first steps
+    branch on it themselves: no quantisation reads anything back to the host.  The host learns of the flag
+    through a copy that it does not wait for (`known_initialised`), and switches to the fused pass once it has;
+    `initialised` is the exact answer and reads the flag if the host does not know yet."""
 
     def __init__(self, dtype: DTypes, history_len: int = DEFAULT_AMAX_HISTORY_LEN, margin: int = DEFAULT_MARGIN,
                  device: Union[str, torch.device] = "cuda"):
@@ -48,7 +53,9 @@ class DelayedScaling:
         # one allocation: [scale, hist[0..H-1]]
         self._buf = torch.zeros(1 + self.history_len, dtype=torch.float32, device=device)
         self._buf[0] = INITIAL_SCALING_FACTOR
-        self.initialised = False
+        self._flag = torch.zeros(1, dtype=torch.float32, device=device)   # 1.0 once a finite positive amax was recorded
+        self._known = False      # the host has seen the flag set
+        self._pending = None     # (pinned host copy of the flag, event behind the copy)
 
     @property
     def scale(self) -> torch.Tensor:
@@ -57,6 +64,41 @@ class DelayedScaling:
     @property
     def amax_history(self) -> torch.Tensor:
         return self._buf[1:]
+
+    @property
+    def known_initialised(self) -> bool:
+        """True once the host has seen the device flag set; never waits.  False may be out of date by a few
+        launches, which only means that the next quantisation still takes the two-launch first-use path."""
+        if not self._known and self._pending is not None:
+            host, event = self._pending
+            if event.query():
+                self._pending = None
+                self._known = bool(host[0] != 0)
+        return self._known
+
+    def _watch_flag(self) -> None:
+        """Queue a copy of the flag to pinned host memory behind the launches issued so far (not under graph capture,
+        where a replay would write into memory the host polls at other times)."""
+        if self._known or self._pending is not None or torch.cuda.is_current_stream_capturing():
+            return
+        host = torch.empty(1, dtype=torch.float32, pin_memory=True)
+        host.copy_(self._flag, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        self._pending = (host, event)
+
+    @property
+    def initialised(self) -> bool:
+        if not self._known:
+            self._pending = None
+            self._known = bool(self._flag.item() != 0)
+        return self._known
+
+    @initialised.setter
+    def initialised(self, value: bool) -> None:
+        self._known = bool(value)
+        self._pending = None
+        self._flag.fill_(1.0 if value else 0.0)
 
     def state_dict(self):
         return {"buf": self._buf.clone(), "initialised": self.initialised}
@@ -145,14 +187,14 @@ def _quantize(cls, tensor: torch.Tensor, dtype: DTypes, state: Optional[DelayedS
         assert state.dtype == dtype, "delayed-scaling state was created for another format"
         assert state._buf.device == dev
         state_p = state._buf.data_ptr()   # [scale, hist[0..H-1]]
-        if not state.initialised:
-            nt.check(nt.lib.ntfp8_quantize_current(x.data_ptr(), xd, rows, cols, fmt, state.margin, amax_p,
-                                                   scale_p, out.data_ptr(), nt.ptr(out_t),
-                                                   state_p + 4, state.history_len, state_p, ws.data_ptr(), st),
-                     "ntfp8_quantize_current")
-            # only while the role has never seen a usable amax: one host read to learn whether it has now
-            a = float(amax.item())
-            state.initialised = a > 0.0 and a != float("inf")
+        if not state.known_initialised:
+            # two launches that decide on the device: current scaling while the role holds no scale, the held scale once
+            # it does (then with the results of the fused pass below, bit for bit)
+            nt.check(nt.lib.ntfp8_quantize_first_use(x.data_ptr(), xd, rows, cols, fmt, state.margin, state_p, state_p + 4,
+                                                     state.history_len, state._flag.data_ptr(), amax_p, scale_p,
+                                                     out.data_ptr(), nt.ptr(out_t), ws.data_ptr(), st),
+                     "ntfp8_quantize_first_use")
+            state._watch_flag()
         else:
             nt.check(nt.lib.ntfp8_quantize_delayed(x.data_ptr(), xd, rows, cols, fmt, state.margin,
                                                    state_p, state_p + 4, state.history_len, amax_p, scale_p,
@@ -188,7 +230,7 @@ def quantize_delayed_batch(tensors, dtype: DTypes, states, with_transpose) -> li
         keep = []
         for d, i in zip(descs, chunk):
             x, state = tensors[i].detach(), states[i]
-            assert state.initialised and state.dtype == dtype and state._buf.device == dev and x.device == dev
+            assert state.known_initialised and state.dtype == dtype and state._buf.device == dev and x.device == dev
             assert x.dtype in nt.TORCH_TO_NT and x.numel() > 0
             if not x.is_contiguous():
                 x = x.contiguous()

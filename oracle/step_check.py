@@ -7,7 +7,8 @@ gradients every step, the master weights perturbed every step so that the weight
 
 What is compared after every layer of every step, product path (FP8Linear on the GPU) against the CPU oracle:
   * bit-exact: the scale used, the amax, the next scale and the whole amax history of the three tensor roles
-    (input e4m3, weight e4m3, output gradient e5m2); the fp8 bytes of the weight and of the quantised input;
+    (input e4m3, weight e4m3, output gradient e5m2); the fp8 bytes of the weight, of the quantised input and of the
+    quantised output gradient;
   * Y and dX (bf16 outputs) on sampled rows against the oracle's fp32 result rounded once to bf16, and dW (fp32,
     optionally added to a pre-filled fp32 master-gradient buffer) on sampled rows against the oracle: rel-L2 <= 1e-3.
 The GEMM semantics follow src/nanotron/fp8/linear.py:69-112 (forward X.W^T; backward dY.W and dY^T.X) and
@@ -71,18 +72,22 @@ def _bits(t: torch.Tensor) -> torch.Tensor:
 
 def check_layer(tag: str, lin, ref: Dict[str, O.DelayedScaling], x: torch.Tensor, w: torch.Tensor, gy: torch.Tensor,
                 y_gpu: torch.Tensor, dx_gpu: torch.Tensor, dw_gpu: torch.Tensor, xq_gpu, step: int, i: int,
-                dw_base: torch.Tensor = None) -> dict:
+                dw_base: torch.Tensor = None, gq_gpu=None) -> dict:
     """Advances the oracle's three roles of this layer by one step and compares; raises AssertionError naming what
     differs.  `xq_gpu` is the FP8Tensor of the input that the layer saved for its backward; `dw_base` (CPU, fp32) is
     what the weight-gradient buffer held before this backward when the layer accumulates into it
-    (src/nanotron/optim/gradient_accumulator.py:222)."""
+    (src/nanotron/optim/gradient_accumulator.py:222); `gq_gpu` is the FP8Tensor of the output gradient that the backward
+    GEMMs read (src/nanotron/fp8/linear.py:99-102), compared like the input when given."""
     xq, wq, gq = ref["input"].quantise(x), ref["weight"].quantise(w), ref["output_grad"].quantise(gy)
     for role, q in (("input", xq), ("weight", wq), ("output_grad", gq)):
         st, rf = lin.scaling[role], ref[role]
         assert torch.equal(_bits(st.scale), _bits(rf.scale)), f"{tag} {role}: next scale {st.scale.item()} != {rf.scale.item()}"
         assert torch.equal(_bits(st.amax_history), _bits(rf.hist)), f"{tag} {role}: amax history differs"
     wg = lin.weight.data
-    for name, got, q in (("weight", wg, wq), ("input", xq_gpu, xq)):
+    operands = [("weight", wg, wq), ("input", xq_gpu, xq)]
+    if gq_gpu is not None:
+        operands.append(("output gradient", gq_gpu, gq))
+    for name, got, q in operands:
         assert torch.equal(_bits(got.fp8_meta.amax), _bits(q.amax)), f"{tag} {name}: amax {got.fp8_meta.amax.item()} != {q.amax.item()}"
         assert torch.equal(_bits(got.fp8_meta.scale), _bits(q.scale)), f"{tag} {name}: scale used {got.fp8_meta.scale.item()} != {q.scale.item()}"
         same = torch.equal(got.as_subclass(torch.Tensor), q.q.to(got.device))

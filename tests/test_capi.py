@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(nt.lib, n), f"{n} declared in include/ntfp8.h but not exported"
         assert n in nt.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(nt.SIGNATURES) == names
-    assert nt.version() == 2
+    assert nt.version() == 3
     assert nt.strerror(0) == "ok" and "NULL" in nt.strerror(-1)
 
 
@@ -224,6 +224,19 @@ def test_new_entry_points_validate_on_the_host():
     assert call(n=0) == -3 and call(hl=0) == -3
     assert call(s1=P + 4202) == -4
     assert call(s1=P + 4096) == -7 and call(o1=P + 8192 + 16) == -7 and call(o0=P + 8) == -7
+    # the first use of a delayed-scaling role, decided on the device
+    args = dict(x=P, x_dtype=2, rows=4, cols=16, fmt=0, margin=0, state=P + 4096, hist=P + 4100, hl=16, flag=P + 4300,
+                amax=P + 4400, used=P + 4404, out=P + 8192, out_t=None, ws=P + 16384)
+    call = lambda **kw: L.ntfp8_quantize_first_use(*[{**args, **kw}[k] for k in args], None)
+    assert call(flag=None) == -1 and call(used=None) == -1 and call(ws=None) == -1 and call(out=None) == -1
+    assert call(hl=0) == -3 and call(rows=0) == -3 and call(margin=200) == -3
+    assert call(fmt=2) == -2 and call(x_dtype=5) == -2
+    assert call(flag=P + 4302) == -4
+    assert call(out=P + 8) == -7
+    # the bandwidth yardstick
+    assert L.ntfp8_stream_probe(0, None, 64, P, None) == -1 and L.ntfp8_stream_probe(3, P, 64, P + 4096, None) == -2
+    assert L.ntfp8_stream_probe(1, P, 48, P + 4096, None) == -3 and L.ntfp8_stream_probe(1, P + 8, 64, P + 4096, None) == -4
+    assert L.ntfp8_stream_probe(2, P, 64, P + 32, None) == -7
 
 
 def test_host_policy_for_transposed_copies():

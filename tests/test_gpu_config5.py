@@ -27,6 +27,7 @@ def _build(linears, accumulate=False):
                         amax_history_len=16, margin=0, accumulate_grad=accumulate)
         w = C.initial_weight(i, K, N)
         lin.weight = FP8Parameter(w.cuda(), DTypes.FP8E4M3)
+        lin.keep_quantised_grad = True   # the checker compares the e5m2 bytes of dY too
         mods.append(lin)
         ws.append(w)
     return mods, ws
@@ -59,7 +60,7 @@ def test_config5_llama3_8b_block_full_size_10_steps():
             y.backward(gy.cuda())
             assert lin.weight.grad is None   # bf16 master: the fp32 gradient lives in main_grad
             errs = C.check_layer(f"step {step} {name}", lin, refs[i], x, ws[i], gy, y.detach(), xg.grad,
-                                 lin.weight.main_grad, xq_gpu, step, i)
+                                 lin.weight.main_grad, xq_gpu, step, i, gq_gpu=lin.quantised_grad_output)
             for k, v in errs.items():
                 worst[k] = max(worst[k], v)
         _say(f"config 5 step {step}: ok, worst rel-L2 so far {worst}")
@@ -93,6 +94,74 @@ def test_config3_and_4_llama7b_mlp_through_fp8linear():
             y.backward(gy.cuda())
             assert lin.weight.main_grad.data_ptr() == buf.data_ptr()   # accumulated in place
             C.check_layer(f"step {step} {name}", lin, refs[i], x, ws[i], gy, y.detach(), xg.grad, lin.weight.main_grad,
-                          xq_gpu, step, i, dw_base=base[i])
+                          xq_gpu, step, i, dw_base=base[i], gq_gpu=lin.quantised_grad_output)
             base[i] = lin.weight.main_grad.cpu()
         _say(f"configs 3/4 step {step}: ok")
+
+
+def test_config5_step_replayed_as_a_graph_matches_eager_launches():
+    """The benchmark step at its real shapes captured once as a HIP graph (weight re-quantisation, then for every
+    linear: quantise X, forward GEMM, quantise dY, dgrad + wgrad launch) and replayed eight times with fresh inputs
+    copied into its static buffers, against an eager twin: outputs, gradients, fp8 weight bytes and the whole scaling
+    state bit for bit after every replay, with eager work and synchronisations between the replays."""
+    from nanotron_amd.fp8.optim import requantize_fp8_weights
+
+    g_mods, ws = _build(C.LINEARS)
+    e_mods, _ = _build(C.LINEARS)
+    sx = [torch.zeros(C.TOKENS, K, dtype=torch.bfloat16, device="cuda", requires_grad=True) for _, K, _ in C.LINEARS]
+    sgy = [torch.zeros(C.TOKENS, N, dtype=torch.bfloat16, device="cuda") for _, _, N in C.LINEARS]
+
+    def load(step):
+        """This step's weights into both sets of modules, its inputs into the static buffers; returns the inputs."""
+        ins = []
+        for i, (name, K, N) in enumerate(C.LINEARS):
+            ws[i] = C.perturbed_weight(ws[i], step, i)
+            w = ws[i].cuda()
+            x, gy = C.step_inputs(step, i, K, N)
+            x, gy = x.cuda(), gy.cuda()
+            with torch.no_grad():
+                g_mods[i].weight.as_subclass(torch.Tensor).copy_(w)
+                e_mods[i].weight.as_subclass(torch.Tensor).copy_(w)
+                sx[i].copy_(x)
+                sgy[i].copy_(gy)
+            ins.append((x, gy))
+        return ins
+
+    def run(mods, xs, gys):
+        requantize_fp8_weights(mods)
+        ys = []
+        for lin, x, gy in zip(mods, xs, gys):
+            x.grad = None
+            y = lin(x)
+            y.backward(gy)
+            ys.append(y)
+        return ys
+
+    side = torch.cuda.Stream()
+    for step in range(2):   # every role gets its first scale (a role's first quantisation reads its amax on the host)
+        ins = load(step)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            run(g_mods, sx, sgy)
+        torch.cuda.current_stream().wait_stream(side)
+        run(e_mods, [x.requires_grad_(True) for x, _ in ins], [gy for _, gy in ins])
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_ys = run(g_mods, sx, sgy)
+    for step in range(2, 10):
+        ins = load(step)
+        graph.replay()
+        xe = [x.requires_grad_(True) for x, _ in ins]
+        e_ys = run(e_mods, xe, [gy for _, gy in ins])
+        _ = float((e_ys[1][:64].float() @ e_ys[1][:64].float().t()).sum())   # unrelated eager work and a synchronisation
+        for i, (name, _, _) in enumerate(C.LINEARS):
+            tag = f"step {step} {name}"
+            assert torch.equal(g_ys[i], e_ys[i]), f"{tag}: Y of the replay differs"
+            assert torch.equal(sx[i].grad, xe[i].grad), f"{tag}: dX of the replay differs"
+            assert torch.equal(g_mods[i].weight.main_grad, e_mods[i].weight.main_grad), f"{tag}: dW of the replay differs"
+            assert torch.equal(g_mods[i].weight.data.as_subclass(torch.Tensor),
+                               e_mods[i].weight.data.as_subclass(torch.Tensor)), f"{tag}: fp8 weight bytes differ"
+            for role in C.ROLES:
+                assert torch.equal(g_mods[i].scaling[role]._buf, e_mods[i].scaling[role]._buf), f"{tag} {role}: scaling state differs"
+        _say(f"config 5 graph replay, step {step}: identical to the eager launches")

@@ -259,6 +259,46 @@ def test_delayed_scaling_zero_first_then_values(fmt):
 
 
 @pytest.mark.parametrize("fmt", FMTS)
+def test_first_use_entry_point_decides_on_the_device(fmt):
+    """ntfp8_quantize_first_use: a role without a scale is scaled from its own amax (src/nanotron/fp8/tensor.py:25-28),
+    a role with one casts with it, and which of the two it is is a flag in device memory that the kernels read and set
+    themselves.  A sequence that holds the flag down for three steps (zeros, NaN, Inf) and then sets it, every step
+    against the oracle's state machine bit for bit, without the host reading anything in between."""
+    from nanotron_amd import _native as nt
+
+    dev = torch.device("cuda")
+    H = 4
+    state = torch.zeros(1 + H, device=dev)
+    state[0] = 1.0
+    flag = torch.zeros(1, device=dev)
+    ref = O.DelayedScaling(fmt, history_len=H, margin=0)
+    g = torch.Generator().manual_seed(5)
+    seq = [torch.zeros(48, 80), torch.full((48, 80), float("nan")), torch.full((48, 80), float("inf")),
+           torch.randn(48, 80, generator=g) * 3, torch.randn(48, 80, generator=g) * 300, torch.zeros(48, 80),
+           torch.randn(48, 80, generator=g) * 0.01, torch.randn(48, 80, generator=g)]
+    seq[2][1:] = 1.0
+    results = []
+    ws, st = nt.workspace_and_stream(dev)
+    for x in seq:
+        xg = x.to(torch.bfloat16).to(dev)
+        out = torch.empty(48, 80, dtype=torch.uint8, device=dev)
+        sc = torch.empty(2, device=dev)
+        nt.check(nt.lib.ntfp8_quantize_first_use(xg.data_ptr(), nt.BF16, 48, 80, nt.E4M3 if fmt == O.E4M3 else nt.E5M2, 0,
+                                                 state.data_ptr(), state.data_ptr() + 4, H, flag.data_ptr(), sc.data_ptr(),
+                                                 sc.data_ptr() + 4, out.data_ptr(), None, ws.data_ptr(), st), "first_use")
+        results.append((xg, out, sc, state.clone(), flag.clone()))
+    for i, (x, (xg, out, sc, stt, fl)) in enumerate(zip(seq, results)):
+        want = ref.quantise(x.to(torch.bfloat16))
+        assert same_float(sc[0].item(), want.amax.item()), i
+        assert sc[1].item() == want.scale.item(), i
+        assert stt[0].item() == ref.scale.item(), i
+        h, hr = stt[1:].cpu(), ref.hist
+        assert torch.equal(torch.isnan(h), torch.isnan(hr)) and torch.equal(h.nan_to_num(-1), hr.nan_to_num(-1)), i
+        assert torch.equal(out.cpu(), want.q), i
+        assert bool(fl.item() != 0) == ref.initialised, i
+
+
+@pytest.mark.parametrize("fmt", FMTS)
 def test_config2_full_size_20_steps(fmt):
     """Benchmark config 2: bf16 [4096,4096] Student-t + outliers, history 16, 20 steps."""
     _, _, DelayedScaling, FP8Tensor, _ = _api()

@@ -186,3 +186,49 @@ def test_step_replayed_as_a_graph_matches_eager():
                                le.weight.main_grad if le.weight.dtype != torch.float32 else le.weight.grad)
             for role in lg.scaling:
                 assert torch.equal(lg.scaling[role]._buf, le.scaling[role]._buf)
+
+
+def test_a_fresh_layers_first_steps_replay_as_a_graph():
+    """No quantisation reads anything back to the host, not even a role's first (which scales from the tensor's own
+    amax and is told apart from the later ones by a flag in device memory): a step captured on layers that have never
+    run replays as their first, second and third step, bit for bit like an eager twin's."""
+    from nanotron_amd.fp8 import FP8Linear
+    from nanotron_amd.fp8.optim import requantize_fp8_weights
+
+    def build():
+        torch.manual_seed(23)
+        return nn.Sequential(FP8Linear(256, 384, bias=False, device="cuda", delayed_scaling=True, out_dtype=torch.bfloat16),
+                             FP8Linear(384, 256, bias=False, device="cuda", delayed_scaling=True, out_dtype=torch.bfloat16))
+
+    def step(model, x, gy):
+        requantize_fp8_weights(model)
+        x.grad = None
+        y = model(x)
+        y.backward(gy)
+        return y
+
+    g_model, e_model = build(), build()
+    sx = torch.zeros(320, 256, dtype=torch.bfloat16, device="cuda", requires_grad=True)
+    sgy = torch.zeros(320, 256, dtype=torch.bfloat16, device="cuda")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        sy = step(g_model, sx, sgy)
+    for i in range(3):
+        x = O.normal_tensor(500 + i, (320, 256), 1.0 + i, torch.bfloat16).cuda()
+        gy = O.normal_tensor(600 + i, (320, 256), 1e-3, torch.bfloat16).cuda()
+        with torch.no_grad():
+            sx.copy_(x)
+            sgy.copy_(gy)
+        graph.replay()
+        xe = x.clone().requires_grad_(True)
+        ye = step(e_model, xe, gy)
+        torch.cuda.synchronize()
+        assert torch.equal(sy, ye), i
+        assert torch.equal(sx.grad, xe.grad), i
+        for lg, le in zip(g_model, e_model):
+            assert torch.equal(lg.weight.grad, le.weight.grad), i
+            for role in lg.scaling:
+                assert torch.equal(lg.scaling[role]._buf, le.scaling[role]._buf), (i, role)
+                assert torch.equal(lg.scaling[role]._flag, le.scaling[role]._flag), (i, role)
+    assert all(st.initialised for lg in g_model for st in lg.scaling.values())
