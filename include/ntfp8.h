@@ -157,9 +157,10 @@ int ntfp8_quantize_delayed_batch(const ntfp8_quant_desc* tensors, int count, voi
  * count above NTFP8_STATIC_MAX_TENSORS returns NTFP8_ERR_SIZE.  Nothing is allocated or freed, here or in any
  * routine it calls.  All calls on one GPU share that GPU's array: calls that may overlap in time (different
  * streams, different threads) race; order them, or use ntfp8_quantize_delayed_batch with workspaces of their own.
- * The per-device address of the array is resolved at the first call on a device (a host-side look-up plus one
- * small clearing kernel on `stream`); ntfp8_static_init does that ahead of time for the current device, e.g. before
- * a graph capture begins. */
+ * The per-device address of the array is resolved at the first call on a device (a host-side look-up, nothing is
+ * launched: the array starts zeroed with the device image and every kernel leaves its workspace zero);
+ * ntfp8_static_init does that ahead of time for the current device, e.g. before a graph capture begins (`stream` is
+ * not used). */
 #define NTFP8_STATIC_MAX_TENSORS 16
 int ntfp8_static_init(void* stream);
 int ntfp8_quantize_delayed_batch_static(const ntfp8_quant_desc* tensors, int count, void* stream);

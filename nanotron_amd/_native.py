@@ -19,6 +19,7 @@ F32, F16, BF16 = 0, 1, 2
 OUT_E4M3, OUT_E5M2 = 3, 4  # d_dtype of an fp8 GEMM output
 WORKSPACE_BYTES = 2048
 STATIC_MAX_TENSORS = 16  # tensors per ntfp8_quantize_delayed_batch_static call
+ERR_UNSUPPORTED, ERR_LAUNCH = -5, -6
 
 TORCH_TO_NT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
@@ -88,6 +89,11 @@ def strerror(code: int) -> str:
 
 def check(code: int, what: str) -> None:
     if code != 0:
+        if code == ERR_LAUNCH:
+            # whatever went wrong at the launch, nothing may be assumed about the reduction workspaces any more (they
+            # must be all zero between launches): drop them, the next call gets fresh zeroed ones
+            _workspaces.clear()
+            _pools.clear()
         raise RuntimeError(f"{what} failed: {strerror(code)} (code {code})")
 
 

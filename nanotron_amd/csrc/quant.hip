@@ -793,26 +793,17 @@ int run_quant_dual(const void* x, int x_dtype, int64_t n, uint8_t* out_e4m3, uin
 // host-side handle of it, the address comes from hipGetSymbolAddress with that device current.
 static __device__ __align__(256) unsigned char scratch[NTFP8_STATIC_MAX_TENSORS * NTFP8_WORKSPACE_BYTES];
 
-__global__ void fill_zero_kernel(uint32_t* p, int words) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < words) p[i] = 0u;
-}
-
-// Device address of `scratch` on the current device, resolved (and the array cleared, on `st`) at the first call
-// for that device.
-int static_scratch(void** out, hipStream_t st) {
+// Device address of `scratch` on the current device, resolved at the first call for that device.  Nothing is launched:
+// a device image starts with the array zeroed and every kernel leaves its workspace zero, so there is nothing to
+// clear, and a clearing kernel on the first caller's stream would race with a first user on another stream.
+int static_scratch(void** out, hipStream_t) {
     static std::atomic<void*> cached[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return NTFP8_ERR_LAUNCH;
     void* p = cached[dev].load(std::memory_order_acquire);
     if (p == nullptr) {
+        // (threads that race here resolve the same address)
         if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return NTFP8_ERR_LAUNCH;
-        // a loaded image starts zeroed and every kernel leaves its workspace zero; cleared once more here so that
-        // the first user does not depend on the loader
-        constexpr int words = NTFP8_STATIC_MAX_TENSORS * NTFP8_WORKSPACE_BYTES / 4;
-        clear_stale_error();
-        hipLaunchKernelGGL(fill_zero_kernel, dim3((words + 255) / 256), dim3(256), 0, st, static_cast<uint32_t*>(p), words);
-        if (hipGetLastError() != hipSuccess) return NTFP8_ERR_LAUNCH;
         cached[dev].store(p, std::memory_order_release);
     }
     *out = p;

@@ -20,6 +20,18 @@ class FP8LinearMeta(TypedDict):
     output_grad: FP8Meta
 
 
+class _GradBox:
+    """What travels beside the autograd graph between an FP8Linear with an fp8 output and the layer that consumes it:
+    the delayed-scaling role the producer quantises its output gradient with, and, during a backward pass, that
+    gradient already as e5m2 bytes out of the consumer's dgrad epilogue (autograd itself only carries a placeholder
+    then: a gradient must have its tensor's type, and the tensor it stands for is the high-precision handle)."""
+
+    __slots__ = ("state", "fp8_grad", "arrivals")
+
+    def __init__(self, state):
+        self.state, self.fp8_grad, self.arrivals = state, None, 0
+
+
 class FP8Linear(nn.Linear):
     """nn.Linear whose matmuls run in FP8 (reference: src/nanotron/fp8/linear.py:24-66).
 
@@ -52,6 +64,12 @@ class FP8Linear(nn.Linear):
         # reference drops it (linear.py:102) and it would pin the bytes until the next backward
         self.keep_quantised_grad = False
         self.quantised_grad_output = None
+        # True: the gradient of an fp8 input that another FP8Linear produced goes back to that layer as e5m2 bytes
+        # straight from this layer's dgrad epilogue (cast with the producer's output-gradient scale) instead of as a
+        # high-precision tensor the producer then quantises
+        self.fp8_grad_input = True
+        self.fp8_grad_inputs_sent = 0   # backward passes of this layer that did so
+        self._grad_box = None
         self.scaling = None
         self._weight_ready = None
         if self.weight.device != torch.device("cpu"):
@@ -179,10 +197,18 @@ class FP8Linear(nn.Linear):
         # The bias goes into the GEMM's epilogue (the TODO at linear.py:62; for the fp32 output of the reference the
         # result equals `output + self.bias`, linear.py:65, bit for bit) and an fp8 input produced by another
         # FP8Linear brings the handle its gradient travels through (below).
-        output, aux = _FP8Matmul.apply(input, self.weight, self.fp8_meta, phony, self, self.bias,
-                                       getattr(input, "_grad_handle", None))
+        handle = getattr(input, "_grad_handle", None)
+        if handle is None and torch.is_grad_enabled() and getattr(getattr(input, "fp8_meta", None), "from_fp8_linear", False):
+            # the bytes of another FP8Linear's output, but not the object it returned (a view, a copy or a slice with
+            # the meta carried over): the producer would silently get no gradient
+            raise RuntimeError("this fp8 activation was produced by an FP8Linear but has lost the gradient handle that "
+                               "layer attached to its output (`_grad_handle`): pass the output object itself, or carry "
+                               "the attribute over to the tensor derived from it")
+        output, aux = _FP8Matmul.apply(input, self.weight, self.fp8_meta, phony, self, self.bias, handle)
         if isinstance(self.out_dtype, DTypes):
             output._grad_handle = aux
+            aux._grad_box = self._grad_box   # made by this forward: where a consuming layer leaves an fp8 gradient
+            output.fp8_meta.from_fp8_linear = True   # travels with the meta if a caller re-wraps the bytes
         return output
 
 
@@ -213,6 +239,7 @@ class _FP8Matmul(torch.autograd.Function):
         ctx.in_dtype = input.dtype if type(input) == torch.Tensor else (input_handle.dtype if input_handle is not None else None)
         ctx.in_shape = input.shape
         ctx.has_handle = input_handle is not None
+        ctx.input_box = getattr(input_handle, "_grad_box", None) if input_handle is not None else None
         if type(input) == torch.Tensor:
             x2d = input.reshape(-1, input.shape[-1])
             input = FP8Tensor(x2d, dtype=DTypes.FP8E4M3, state=scaling["input"] if scaling else None,
@@ -235,6 +262,7 @@ class _FP8Matmul(torch.autograd.Function):
                 out_dtype=out_dtype, out_state=state, out_with_transpose=module.fp8_output_transpose, bias=gemm_bias,
             )
             ctx.mark_non_differentiable(output)
+            ctx.grad_box = module._grad_box = _GradBox(scaling["output_grad"] if scaling else None)
             hp = weight.dtype if weight.dtype in (torch.float32, torch.float16, torch.bfloat16) else torch.float32
             handle = torch.zeros(1, dtype=hp, device=output.device).expand(output.shape)
             ctx.fp8_out = True
@@ -256,7 +284,17 @@ class _FP8Matmul(torch.autograd.Function):
         scaling = module.scaling if module is not None else None
         none = (None,) * 7
         if ctx.fp8_out:
-            grad_output = grad_aux   # the gradient of the fp8 output arrives through its handle
+            grad_output = grad_aux   # the gradient of the fp8 output arrives through its handle ...
+            box = ctx.grad_box
+            fp8_grad, arrivals = box.fp8_grad, box.arrivals
+            box.fp8_grad, box.arrivals = None, 0
+            if fp8_grad is not None:
+                if arrivals > 1:
+                    raise RuntimeError("an fp8 activation with more than one consumer received a gradient in fp8 from one of "
+                                       "them: fp8 contributions cannot be summed.  Set `fp8_grad_input = False` on the "
+                                       "consuming FP8Linears (high-precision gradients, summed by autograd), or give the "
+                                       "producing layer a high-precision out_dtype")
+                grad_output = fp8_grad   # ... or beside it, already quantised by the consumer's dgrad epilogue
         if grad_output is None:
             return none
 
@@ -279,11 +317,16 @@ class _FP8Matmul(torch.autograd.Function):
                 x_plain and a_transposed_supported(g2d.shape[1], input.shape[1], g2d.shape[0]))
             grad_output = FP8Tensor(g2d, dtype=DTypes.FP8E5M2, state=scaling["output_grad"] if scaling else None,
                                     with_transpose=with_t)
-            if module is not None and module.keep_quantised_grad:
-                module.quantised_grad_output = grad_output   # for checkers: the e5m2 operand of dgrad and wgrad
+        if module is not None and module.keep_quantised_grad:
+            module.quantised_grad_output = grad_output   # for checkers: the e5m2 operand of dgrad and wgrad
 
         wants_dx = ctx.needs_input_grad[0] or (ctx.has_handle and ctx.needs_input_grad[6])
         grad_input = None
+        box = ctx.input_box if wants_dx else None
+        if box is not None:
+            box.arrivals += 1
+        fp8_dx = (box is not None and box.arrivals == 1 and box.state is not None and box.state.known_initialised
+                  and module is not None and module.fp8_grad_input)
         # dX[M,K] = dY[M,N] . W[N,K]
         dgrad = dict(mat_a=weight.data, transpose_a=False, mat_b=grad_output, transpose_b=False, use_split_accumulator=True,
                      out_dtype=ctx.in_dtype or torch.float32)
@@ -301,7 +344,17 @@ class _FP8Matmul(torch.autograd.Function):
             wgrad = dict(mat_a=input, transpose_a=False, mat_b=grad_output, transpose_b=True, use_split_accumulator=True,
                          accumulate_into=acc)
         grad_weight = None
-        if wants_dx and wgrad is not None:
+        if fp8_dx:
+            # dX leaves the dgrad epilogue as e5m2 bytes under the producer's output-gradient role (amax, history roll and
+            # next scale included: what the producer's own quantisation of a high-precision dX would have done, minus
+            # the rounding to the high-precision type in between); autograd carries a placeholder without memory
+            box.fp8_grad = fp8_matmul_kernel(mat_a=weight.data, transpose_a=False, mat_b=grad_output, transpose_b=False,
+                                             use_split_accumulator=True, out_dtype=DTypes.FP8E5M2, out_state=box.state)
+            grad_input = torch.zeros(1, dtype=ctx.in_dtype or torch.float32, device=grad_output.device).expand(ctx.in_shape)
+            module.fp8_grad_inputs_sent += 1
+            if wgrad is not None:
+                grad_weight = fp8_matmul_kernel(**wgrad)
+        elif wants_dx and wgrad is not None:
             # the two GEMMs are independent: issued together they share kernel launches
             grad_input, grad_weight = fp8_matmul_pair(
                 {k: v for k, v in dgrad.items() if k != "use_split_accumulator"},

@@ -115,15 +115,19 @@ def te_gemm(A: torch.Tensor, A_scale_inverse: torch.Tensor, A_type, transa: bool
             math_sm_count: int = 0) -> None:
     """cuBLASLt's column-major GEMM on row-major torch tensors, written into D:
         transa=True,  transb=False:  D[B.rows, A.rows] = B . A^T        (the form the reference issues)
-        transa=False, transb=False:  D[B.rows, A.cols] = B . A          (A is read as it is, no transposed copy)
-        transa=False, transb=True:   D[B.cols, A.cols] = B^T . A        (both read as they are: the wgrad form)
+        transa=False, transb=False:  D[B.rows, A.cols] = B . A
+        transa=False, transb=True:   D[B.cols, A.cols] = B^T . A        (the wgrad form)
+        transa=True,  transb=True:   D[B.cols, A.rows] = B^T . A^T
     times A_scale_inverse * B_scale_inverse, fp32 accumulation, plus `bias` (one value per column of D) if it is
     not empty, one rounding to D's type; `accumulate` adds into an fp32 D.  With an fp8 `D_type`, D receives
-    sat_rne_fp8(result * D_scale) and D_amax max(D_amax, max|result|).  transa=True with transb=True, `grad` (bias
-    gradient) and a non-empty `pre_gelu_out` are not served.  `workspace`, `use_split_accumulator` and `math_sm_count` have no
-    meaning here: the kernels need no workspace and the matrix cores always accumulate in fp32."""
-    if transb and transa:
-        raise RuntimeError("te_gemm: transa=True with transb=True is not supported")
+    sat_rne_fp8(result * D_scale) and D_amax max(D_amax, max|result|).
+
+    Every form is served for every shape.  The library reads an operand that is not contiguous along the reduction
+    index as it lies in memory where its big kernel can (no bias, N a multiple of 16, M and N above 128, K >= 256,
+    operands below 2 GiB; a transposed B only next to a transposed A); elsewhere the operand is transposed first
+    (ntfp8_transpose) and the K-contiguous form is issued, which has no such limits.  Not served: `grad` together with
+    a bias (the bias-gradient epilogue) and a non-empty `pre_gelu_out`.  `workspace`, `use_split_accumulator` and
+    `math_sm_count` have no meaning here: the kernels need no workspace and the matrix cores always accumulate in fp32."""
     if grad and bias is not None and bias.numel() > 0:
         raise RuntimeError("te_gemm: the bias-gradient epilogue (grad=True with a bias) is not supported")
     if pre_gelu_out is not None and pre_gelu_out.numel() > 0:
@@ -151,10 +155,24 @@ def te_gemm(A: torch.Tensor, A_scale_inverse: torch.Tensor, A_type, transa: bool
     p.B, p.scale_b, p.fmt_b = a.data_ptr(), sa.data_ptr(), _fmt(A_type)
     p.b_transposed = 0 if transa else 1
     p.a_transposed = 1 if transb else 0
+    has_bias = bias is not None and bias.numel() > 0
+    # forms the library does not read in place: transposed copies and the K-contiguous form
+    copies = (p.a_transposed and not p.b_transposed) or (has_bias and (p.a_transposed or p.b_transposed))
+
+    def use_copies():
+        nonlocal a, b
+        if p.b_transposed:
+            a = fp8_transpose(a, A_type)
+        if p.a_transposed:
+            b = fp8_transpose(b, B_type)
+        p.A, p.B, p.a_transposed, p.b_transposed = b.data_ptr(), a.data_ptr(), 0, 0
+        keep.extend([a, b])
     p.scales_are_inverse = 1
     p.D, p.M, p.N, p.K = D.data_ptr(), M, N, K
     p.accumulate = 1 if accumulate else 0
     keep = [a, b, sa, sb]
+    if copies:
+        use_copies()
     st = nt.stream_ptr(dev)
     fp8_out = D.dtype == torch.uint8
     if fp8_out:
@@ -173,13 +191,17 @@ def te_gemm(A: torch.Tensor, A_scale_inverse: torch.Tensor, A_type, transa: bool
         if D.dtype not in nt.TORCH_TO_NT:
             raise RuntimeError(f"te_gemm: unsupported output type {D.dtype}")
         p.d_dtype = nt.TORCH_TO_NT[D.dtype]
-    if bias is not None and bias.numel() > 0:
+    if has_bias:
         if bias.numel() != N or bias.dtype not in nt.TORCH_TO_NT:
             raise RuntimeError(f"te_gemm: bias must hold {N} fp32 / fp16 / bf16 values")
         bb = bias.detach().to(dev).contiguous()
         p.bias, p.bias_dtype = bb.data_ptr(), nt.TORCH_TO_NT[bb.dtype]
         keep.append(bb)
-    nt.check(nt.lib.ntfp8_gemm_batch(d, 1, st), "te_gemm")
+    rc = nt.lib.ntfp8_gemm_batch(d, 1, st)
+    if rc == nt.ERR_UNSUPPORTED and (p.a_transposed or p.b_transposed):
+        use_copies()   # a shape the in-place reads do not serve (refused before anything was launched)
+        rc = nt.lib.ntfp8_gemm_batch(d, 1, st)
+    nt.check(rc, "te_gemm")
     if fp8_out and want_amax:
         # the maxima the epilogue left in the workspace -> max(D_amax, max|result|); no history, scale untouched
         am = D_amax if (D_amax.device == dev and D_amax.dtype == torch.float32) else None

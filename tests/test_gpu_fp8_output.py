@@ -225,6 +225,90 @@ def test_two_linears_chained_through_an_fp8_activation():
     assert "fp8_state.output" in first.state_dict()
 
 
+def test_gradient_of_an_fp8_activation_goes_back_as_fp8_bytes():
+    """Backward of a chain FP8Linear(out fp8) -> FP8Linear: once the producer's output-gradient role holds a scale, the
+    consumer's dgrad epilogue writes dX as e5m2 bytes under that role (the TODO at src/nanotron/fp8/linear.py:63-64,
+    backward direction) and autograd only carries a placeholder.  The bytes, the scale used and the role's state must
+    equal the quantisation of the fp32 dgrad result under the same role; the producer's gradients are then checked
+    against the oracle on those bytes.  A second consumer of the same activation is refused."""
+    from nanotron_amd.fp8 import DTypes, FP8Linear, FP8Parameter, FP8Tensor
+    from nanotron_amd.fp8.kernel import fp8_matmul_kernel
+
+    T, H, I = 384, 256, 512
+    w1 = O.normal_tensor(51, (I, H), 0.05, torch.float32)
+    w2 = O.normal_tensor(52, (H, I), 0.05, torch.float32)
+    first = FP8Linear(H, I, bias=False, device="cuda", out_dtype=DTypes.FP8E4M3, delayed_scaling=True, amax_history_len=4)
+    second = FP8Linear(I, H, bias=False, device="cuda", delayed_scaling=True, amax_history_len=4, out_dtype=torch.bfloat16)
+    for lin, w in ((first, w1), (second, w2)):
+        lin.weight = FP8Parameter(w.cuda(), DTypes.FP8E4M3)
+        lin.keep_quantised_grad = True
+    for step in range(4):
+        x = O.normal_tensor(60 + step, (T, H), 1.0 + 0.5 * step, torch.bfloat16).cuda().requires_grad_(True)
+        gy = O.normal_tensor(70 + step, (T, H), 1e-3 * (1 + step), torch.bfloat16).cuda()
+        role = first.scaling["output_grad"]
+        fp8_path = role.initialised   # (reads the flag: from the second step on)
+        before = _clone_state(role)
+        h = first(x)
+        y = second(h)
+        y.backward(gy)
+        got = first.quantised_grad_output          # what the producer's backward GEMMs read
+        assert isinstance(got, FP8Tensor) and got.fp8_meta.dtype == DTypes.FP8E5M2 and tuple(got.shape) == (T, I)
+        # the fp32 dgrad of the consumer on the operands it used, quantised under the producer's role as it stood
+        dx32 = fp8_matmul_kernel(mat_a=second.weight.data, transpose_a=False, mat_b=second.quantised_grad_output,
+                                 transpose_b=False, use_split_accumulator=True)
+        if fp8_path:
+            want = FP8Tensor(dx32, DTypes.FP8E5M2, state=before)
+            assert torch.equal(got.as_subclass(torch.Tensor), want.as_subclass(torch.Tensor)), step
+            assert _same_f32(got.fp8_meta.scale, want.fp8_meta.scale) and _same_f32(got.fp8_meta.amax, want.fp8_meta.amax), step
+            assert _same_f32(role._buf, before._buf), step
+        else:
+            # through the high-precision handle: rounded to its type (the producer's master-weight type), then quantised
+            want = FP8Tensor(dx32.to(h._grad_handle.dtype), DTypes.FP8E5M2, state=before)
+            assert torch.equal(got.as_subclass(torch.Tensor), want.as_subclass(torch.Tensor)), step
+        # the producer's own gradients from those bytes, against the oracle
+        gq = O.Quantised(got.as_subclass(torch.Tensor).cpu(), got.fp8_meta.amax.cpu(), got.fp8_meta.scale.cpu(), O.E5M2)
+        wq = O.Quantised(first.weight.data.as_subclass(torch.Tensor).cpu(), first.weight.data.fp8_meta.amax.cpu(),
+                         first.weight.data.fp8_meta.scale.cpu(), O.E4M3)
+        assert O.rel_l2(x.grad.float().cpu(), O.linear_dgrad(gq, wq).to(torch.bfloat16).float()) <= 1e-3, step
+        assert first.weight.grad is not None and second.weight.grad is not None
+    # two consumers of one fp8 activation: refused when one of them sends its gradient back in fp8
+    third = FP8Linear(I, H, bias=False, device="cuda", delayed_scaling=True, out_dtype=torch.bfloat16)
+    x = O.normal_tensor(99, (T, H), 1.0, torch.bfloat16).cuda().requires_grad_(True)
+    h = first(x)
+    with pytest.raises(RuntimeError, match="more than one consumer"):
+        (second(h).float().sum() + third(h).float().sum()).backward()
+    # ... and served in high precision when the consumers are told so
+    second.fp8_grad_input = third.fp8_grad_input = False
+    h = first(x)
+    (second(h).float().sum() + third(h).float().sum()).backward()
+    assert x.grad is not None
+
+
+def test_an_fp8_activation_that_lost_its_gradient_handle_is_refused():
+    """The gradient of an fp8 activation travels through the `_grad_handle` attribute of the object the producing layer
+    returned.  A tensor derived from it (here: the same bytes re-wrapped, meta carried over) has no handle; consuming it
+    with autograd on would leave the producer without any gradient, silently, so the consumer refuses."""
+    from nanotron_amd.fp8 import DTypes, FP8Linear, FP8Tensor
+
+    first = FP8Linear(256, 384, bias=False, device="cuda", out_dtype=DTypes.FP8E4M3, delayed_scaling=True)
+    second = FP8Linear(384, 256, bias=False, device="cuda", delayed_scaling=True)
+    x = O.normal_tensor(31, (320, 256), 1.0, torch.bfloat16).cuda().requires_grad_(True)
+    for _ in range(2):   # the output role holds a scale from the second step on (the epilogue path)
+        h = first(x)
+        assert h._grad_handle is not None and h.fp8_meta.from_fp8_linear
+        second(h).float().sum().backward()   # the object itself: fine, the producer gets its gradients
+        assert x.grad is not None and first.weight.grad is not None
+    h = first(x)
+    derived = torch.Tensor._make_subclass(FP8Tensor, h.as_subclass(torch.Tensor).view(320, 384))
+    derived.fp8_meta = h.fp8_meta
+    with pytest.raises(RuntimeError, match="gradient handle"):
+        second(derived)
+    with torch.no_grad():   # without autograd there is nothing to lose
+        second(derived)
+    derived._grad_handle = h._grad_handle   # carried over by the caller: accepted
+    second(derived).float().sum().backward()
+
+
 @pytest.mark.parametrize("fo", FMTS)
 @pytest.mark.parametrize("form", ["dgrad", "wgrad"])
 @pytest.mark.parametrize("shape", [(512, 384, 640), (4096, 1024, 2048), (272, 400, 288)])

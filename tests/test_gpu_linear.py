@@ -127,6 +127,30 @@ def test_linear_fwd_bwd_nonsquare_real_gradients(shape, dtype):
     assert O.rel_l2(lin.weight.grad.cpu(), dw_ref) <= REL_L2
 
 
+def test_fp8matmul_apply_with_the_references_four_arguments():
+    """`_FP8Matmul.apply(input, weight, fp8_meta, phony)` exactly as src/nanotron/fp8/linear.py:60 calls it (no module,
+    no bias, no handle): current scaling, fp32 output; forward, dX and the `weight.grad` side effect against the oracle."""
+    from nanotron_amd.fp8 import DTypes, FP8Linear, FP8Parameter
+    from nanotron_amd.fp8.linear import _FP8Matmul
+
+    M, K, N = 192, 160, 272
+    x = O.normal_tensor(41, (M, K), 1.0, torch.float32)
+    w = O.normal_tensor(42, (N, K), 0.02, torch.float32)
+    gy = O.normal_tensor(43, (M, N), 1e-3, torch.float32)
+    lin = FP8Linear(K, N, bias=False, device="cuda")   # only for its fp8_meta dictionary, as linear.py:33-49 builds it
+    weight = FP8Parameter(w.cuda(), DTypes.FP8E4M3)
+    xg = x.cuda().requires_grad_(True)
+    phony = torch.empty(0, device="cuda", requires_grad=True)
+    output, _ = _FP8Matmul.apply(xg, weight, lin.fp8_meta, phony)
+    assert output.dtype == torch.float32 and output.shape == (M, N)
+    output.backward(gy.cuda())
+    xq, wq, gq, y_ref, dx_ref, dw_ref = _oracle_step(x, w, gy)
+    assert O.rel_l2(output.detach().cpu(), y_ref) <= REL_L2
+    assert O.rel_l2(xg.grad.cpu(), dx_ref) <= REL_L2
+    assert weight.grad.dtype == torch.float32 and O.rel_l2(weight.grad.cpu(), dw_ref) <= REL_L2
+    assert phony.grad is None
+
+
 def test_linear_3d_input_bias_and_out_dtype():
     from nanotron_amd.fp8 import DTypes, FP8Linear, FP8Parameter
 

@@ -159,7 +159,8 @@ def test_the_three_gemms_of_a_linear_layer_through_the_reference_call_site(shape
 
 def test_te_gemm_integer_operands_bit_exact_all_arguments():
     """Integer-valued operands sum exactly in any order: the result must equal the fp64 product bit for bit, with
-    inverse scales that are no powers of two, a bias, accumulation into D, and A read untransposed (transa=False)."""
+    inverse scales that are no powers of two, a bias, accumulation into D, and all four transa / transb forms on
+    shapes the big kernel serves in place (1024 x 512 x 256), ragged ones (300 x 272 x 384) and small ones."""
     tex = _tex()
     g = torch.Generator().manual_seed(5)
     one = torch.tensor(1.0)
@@ -182,21 +183,22 @@ def test_te_gemm_integer_operands_bit_exact_all_arguments():
         tex.te_gemm(aq, sa_inv, tex.DType.kFloat8E4M3, True, bq, sb_inv, tex.DType.kFloat8E5M2, False,
                     D, e, tex.DType.kFloat32, e, torch.tensor([]), tex.DType.kFloat32, e, False, ws, 16, True, True, 0)
         assert torch.equal(D.cpu(), want + 7.0)
-        if M > 128 and N > 128 and K >= 256:
-            at = O.cast_to_fp8(a.t().contiguous(), one, O.E4M3).cuda()   # A as [K, N], read without a transposed copy
+        # every transa / transb form, for every shape: operands read as they lie where the big kernel can, through
+        # transposed copies elsewhere (small or ragged shapes, a bias, transa = transb = True)
+        at = O.cast_to_fp8(a.t().contiguous(), one, O.E4M3).cuda()   # A as [K, N]
+        bt = O.cast_to_fp8(b.t().contiguous(), one, O.E5M2).cuda()   # B as [K, M]
+        for A_, ta, B_, tb in ((at, False, bq, False), (at, False, bt, True), (aq, True, bt, True)):
             D = torch.empty(M, N, device="cuda")
-            tex.te_gemm(at, sa_inv, tex.DType.kFloat8E4M3, False, bq, sb_inv, tex.DType.kFloat8E5M2, False,
+            tex.te_gemm(A_, sa_inv, tex.DType.kFloat8E4M3, ta, B_, sb_inv, tex.DType.kFloat8E5M2, tb,
                         D, e, tex.DType.kFloat32, e, torch.tensor([]), tex.DType.kFloat32, e, False, ws, 16, False, True, 0)
-            assert torch.equal(D.cpu(), want)
-            if M % 16 == 0:
-                bt = O.cast_to_fp8(b.t().contiguous(), one, O.E5M2).cuda()   # B as [K, M] too: the wgrad form, transb=True
-                D = torch.empty(M, N, device="cuda")
-                tex.te_gemm(at, sa_inv, tex.DType.kFloat8E4M3, False, bt, sb_inv, tex.DType.kFloat8E5M2, True,
-                            D, e, tex.DType.kFloat32, e, torch.tensor([]), tex.DType.kFloat32, e, False, ws, 16, False, True, 0)
-                assert torch.equal(D.cpu(), want)
-    with pytest.raises(RuntimeError):
-        tex.te_gemm(aq, sa_inv, tex.DType.kFloat8E4M3, True, bq, sb_inv, tex.DType.kFloat8E5M2, True,
-                    D, e, tex.DType.kFloat32, e, torch.tensor([]), tex.DType.kFloat32, e, False, ws, 16, False, True, 0)
+            assert torch.equal(D.cpu(), want), (M, N, K, ta, tb)
+            D = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+            tex.te_gemm(A_, sa_inv, tex.DType.kFloat8E4M3, ta, B_, sb_inv, tex.DType.kFloat8E5M2, tb,
+                        D, e, tex.DType.kFloat32, e, bias.cuda(), tex.DType.kFloat32, e, False, ws, 16, False, True, 0)
+            assert torch.equal(D.cpu(), (want + bias).to(torch.bfloat16)), (M, N, K, ta, tb, "bias")
+    with pytest.raises(RuntimeError):   # the bias-gradient epilogue is not served
+        tex.te_gemm(aq, sa_inv, tex.DType.kFloat8E4M3, True, bq, sb_inv, tex.DType.kFloat8E5M2, False,
+                    D, e, tex.DType.kFloat32, e, bias.cuda(), tex.DType.kFloat32, e, True, ws, 16, False, True, 0)
 
 
 def test_te_gemm_fp8_output_with_scale_and_amax():

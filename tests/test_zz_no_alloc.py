@@ -26,7 +26,10 @@ def _run(entry, xs, fmt, states, with_t, static):
 
     dev = xs[0].device
     descs = (nt.QuantDesc * len(xs))()
-    pool, st = nt.workspace_pool(dev, len(xs))
+    if static:
+        pool, st = None, nt.stream_ptr(dev)   # no workspaces from the caller
+    else:
+        pool, st = nt.workspace_pool(dev, len(xs))
     keep = []
     for i, (d, x, state, wt) in enumerate(zip(descs, xs, states, with_t)):
         cols = x.shape[-1]
@@ -41,7 +44,14 @@ def _run(entry, xs, fmt, states, with_t, static):
         d.out, d.out_t = out.data_ptr(), nt.ptr(out_t)
         d.workspace = None if static else pool[i].data_ptr()
         keep.append((out, out_t, sc))
+    if static:
+        # the call itself must leave device memory as it found it: outputs exist, the library was initialised
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info(dev)[0]
     nt.check(entry(descs, len(xs), st), "quantize batch")
+    if static:
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info(dev)[0] == free_before, "the entry point that allocates nothing allocated"
     return keep
 
 
