@@ -1029,12 +1029,12 @@ def main():
                          "traffic": traffic["quant"], "traffic_source": traffic["source"], "algorithmic_bytes": qb,
                          "kernel": "quant_flat_kernel", "ms": {k: round(v, 5) for k, v in qms.items()}},
         })
-        probe = stream_probe_ms(bufs, 64)
-        out["roofline"]["frac_of_yardstick"] = round(probe["read_2B_write_1B"] / q_avg, 4)
+        yard = stream_probe_ms(bufs, 64)
+        out["roofline"]["frac_of_yardstick"] = round(yard["read_2B_write_1B"] / q_avg, 4)
         out["yardstick"] = {"what": "ntfp8_stream_probe on the same tensors: same grid and 128-bit streaming accesses, no arithmetic, "
                                     "no reduction",
                             **{k: {"ms": round(v, 5), "GBps": round(b * 4096 * 4096 / (v * 1e-3) / 1e9, 1)}
-                               for (k, v), b in zip(probe.items(), (2.0, 3.0, 4.0))}}
+                               for (k, v), b in zip(yard.items(), (2.0, 3.0, 4.0))}}
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_baseline_quant()
     print(json.dumps(out))
