@@ -24,12 +24,15 @@ class _GradBox:
     """What travels beside the autograd graph between an FP8Linear with an fp8 output and the layer that consumes it:
     the delayed-scaling role the producer quantises its output gradient with, and, during a backward pass, that
     gradient already as e5m2 bytes out of the consumer's dgrad epilogue (autograd itself only carries a placeholder
-    then: a gradient must have its tensor's type, and the tensor it stands for is the high-precision handle)."""
+    then: a gradient must have its tensor's type, and the tensor it stands for is the high-precision handle).
+    `consumers` counts the layers whose forward took the activation with gradients on: fp8 contributions cannot be
+    summed, so the fp8 hand-over is used only while there is exactly one, and an activation with several consumers
+    gets high-precision gradients that autograd sums."""
 
-    __slots__ = ("state", "fp8_grad", "arrivals")
+    __slots__ = ("state", "fp8_grad", "arrivals", "consumers")
 
     def __init__(self, state):
-        self.state, self.fp8_grad, self.arrivals = state, None, 0
+        self.state, self.fp8_grad, self.arrivals, self.consumers = state, None, 0, 0
 
 
 class FP8Linear(nn.Linear):
@@ -66,7 +69,8 @@ class FP8Linear(nn.Linear):
         self.quantised_grad_output = None
         # True: the gradient of an fp8 input that another FP8Linear produced goes back to that layer as e5m2 bytes
         # straight from this layer's dgrad epilogue (cast with the producer's output-gradient scale) instead of as a
-        # high-precision tensor the producer then quantises
+        # high-precision tensor the producer then quantises; the producer's bias gradient is then summed from the
+        # e5m2 values.  Used only while this layer is the activation's one consumer
         self.fp8_grad_input = True
         self.fp8_grad_inputs_sent = 0   # backward passes of this layer that did so
         self._grad_box = None
@@ -204,6 +208,10 @@ class FP8Linear(nn.Linear):
             raise RuntimeError("this fp8 activation was produced by an FP8Linear but has lost the gradient handle that "
                                "layer attached to its output (`_grad_handle`): pass the output object itself, or carry "
                                "the attribute over to the tensor derived from it")
+        if handle is not None and handle.requires_grad and torch.is_grad_enabled():
+            box = getattr(handle, "_grad_box", None)
+            if box is not None:
+                box.consumers += 1
         output, aux = _FP8Matmul.apply(input, self.weight, self.fp8_meta, phony, self, self.bias, handle)
         if isinstance(self.out_dtype, DTypes):
             output._grad_handle = aux
@@ -290,10 +298,10 @@ class _FP8Matmul(torch.autograd.Function):
             box.fp8_grad, box.arrivals = None, 0
             if fp8_grad is not None:
                 if arrivals > 1:
-                    raise RuntimeError("an fp8 activation with more than one consumer received a gradient in fp8 from one of "
-                                       "them: fp8 contributions cannot be summed.  Set `fp8_grad_input = False` on the "
-                                       "consuming FP8Linears (high-precision gradients, summed by autograd), or give the "
-                                       "producing layer a high-precision out_dtype")
+                    raise RuntimeError("an fp8 activation received gradients from more than one backward pass of its consumers, "
+                                       "one of them in fp8: fp8 contributions cannot be summed.  Set `fp8_grad_input = False` "
+                                       "on the consuming FP8Linear (high-precision gradients, summed by autograd), or give "
+                                       "the producing layer a high-precision out_dtype")
                 grad_output = fp8_grad   # ... or beside it, already quantised by the consumer's dgrad epilogue
         if grad_output is None:
             return none
@@ -325,8 +333,8 @@ class _FP8Matmul(torch.autograd.Function):
         box = ctx.input_box if wants_dx else None
         if box is not None:
             box.arrivals += 1
-        fp8_dx = (box is not None and box.arrivals == 1 and box.state is not None and box.state.known_initialised
-                  and module is not None and module.fp8_grad_input)
+        fp8_dx = (box is not None and box.consumers == 1 and box.arrivals == 1 and box.state is not None
+                  and box.state.known_initialised and module is not None and module.fp8_grad_input)
         # dX[M,K] = dY[M,N] . W[N,K]
         dgrad = dict(mat_a=weight.data, transpose_a=False, mat_b=grad_output, transpose_b=False, use_split_accumulator=True,
                      out_dtype=ctx.in_dtype or torch.float32)

@@ -230,7 +230,7 @@ def test_gradient_of_an_fp8_activation_goes_back_as_fp8_bytes():
     consumer's dgrad epilogue writes dX as e5m2 bytes under that role (the TODO at src/nanotron/fp8/linear.py:63-64,
     backward direction) and autograd only carries a placeholder.  The bytes, the scale used and the role's state must
     equal the quantisation of the fp32 dgrad result under the same role; the producer's gradients are then checked
-    against the oracle on those bytes.  A second consumer of the same activation is refused."""
+    against the oracle on those bytes.  With a second consumer of the same activation both send high-precision gradients."""
     from nanotron_amd.fp8 import DTypes, FP8Linear, FP8Parameter, FP8Tensor
     from nanotron_amd.fp8.kernel import fp8_matmul_kernel
 
@@ -271,17 +271,37 @@ def test_gradient_of_an_fp8_activation_goes_back_as_fp8_bytes():
                          first.weight.data.fp8_meta.scale.cpu(), O.E4M3)
         assert O.rel_l2(x.grad.float().cpu(), O.linear_dgrad(gq, wq).to(torch.bfloat16).float()) <= 1e-3, step
         assert first.weight.grad is not None and second.weight.grad is not None
-    # two consumers of one fp8 activation: refused when one of them sends its gradient back in fp8
+    # two consumers of one fp8 activation: fp8 contributions cannot be summed, so both send high-precision gradients that
+    # autograd sums on the handle, and nothing goes back as fp8
     third = FP8Linear(I, H, bias=False, device="cuda", delayed_scaling=True, out_dtype=torch.bfloat16)
     x = O.normal_tensor(99, (T, H), 1.0, torch.bfloat16).cuda().requires_grad_(True)
-    h = first(x)
-    with pytest.raises(RuntimeError, match="more than one consumer"):
+    sent = (second.fp8_grad_inputs_sent, third.fp8_grad_inputs_sent)
+    for _ in range(3):   # (these gradients are far larger than the steps' above: let the delayed scales of both levels settle)
+        x.grad = None
+        h = first(x)
         (second(h).float().sum() + third(h).float().sum()).backward()
-    # ... and served in high precision when the consumers are told so
+    assert (second.fp8_grad_inputs_sent, third.fp8_grad_inputs_sent) == sent
+    both = x.grad.float().clone()
+    assert bool(torch.isfinite(both).all()) and float(both.abs().max()) > 0
+    # ... the same as with the fp8 hand-over switched off by hand
     second.fp8_grad_input = third.fp8_grad_input = False
+    for lin in (first, second, third):
+        lin.train(False)     # evaluation mode: the scaling roles stay as they are, so the two passes are comparable
+    x.grad = None
     h = first(x)
     (second(h).float().sum() + third(h).float().sum()).backward()
-    assert x.grad is not None
+    by_hand = x.grad.float().clone()
+    second.fp8_grad_input = third.fp8_grad_input = True
+    x.grad = None
+    h = first(x)
+    (second(h).float().sum() + third(h).float().sum()).backward()
+    assert torch.equal(x.grad.float(), by_hand)
+    # one consumer again: back to fp8
+    for lin in (first, second, third):
+        lin.train(True)
+    h = first(x)
+    second(h).float().sum().backward()
+    assert second.fp8_grad_inputs_sent == sent[0] + 1
 
 
 def test_an_fp8_activation_that_lost_its_gradient_handle_is_refused():
