@@ -42,18 +42,23 @@ __device__ int g_plain_tile_order = 0;
 // build are wrong, only its stamps mean something).  -DNTFP8_KNOCKOUT=<bits> leaves parts of the loop out: 1 the global
 // loads (stale registers are deposited), 2 the deposits into LDS, 4 the workgroup barrier, 8 the LDS reads of the B
 // fragments, 16 those of the A fragments.  -DNTFP8_IDLE=<n> lets every wave sleep 64 n cycles behind the barrier of
-// every K-tile.
+// every K-tile.  -DNTFP8_COLUMNS=<6 | 7> runs the K loop of a tile that is 192 or 224 columns wide instead of 256 (that
+// many of a wave's eight block columns, B loads and B fragments; the schedule is the same with the last front groups
+// left out): what a tile width that divides N = 6144 or 14336 into a whole number of rounds would cost per K-tile.
 #ifndef NTFP8_KNOCKOUT
 #define NTFP8_KNOCKOUT 0
 #endif
 #ifndef NTFP8_IDLE
 #define NTFP8_IDLE 0
 #endif
-constexpr int kKnockout = NTFP8_KNOCKOUT, kIdle = NTFP8_IDLE;
+#ifndef NTFP8_COLUMNS
+#define NTFP8_COLUMNS 8
+#endif
+constexpr int kKnockout = NTFP8_KNOCKOUT, kIdle = NTFP8_IDLE, kColumns = NTFP8_COLUMNS;
 #else
 #define NTFP8_STAMP(var) (void)0
 #define NTFP8_CYCLES(var) (void)0
-constexpr int kKnockout = 0, kIdle = 0;
+constexpr int kKnockout = 0, kIdle = 0, kColumns = 8;
 #endif
 constexpr bool kNoLoads = kKnockout & 1, kNoDeposits = kKnockout & 2, kNoBarrier = kKnockout & 4, kNoBReads = kKnockout & 8,
                kNoAReads = kKnockout & 16;
@@ -385,9 +390,10 @@ void gemm_nt_big_kernel(const BigLaunch L) {
     const float alpha = descale_factor(P.scale_a, P.scale_b, P.ex.scale_inv);
 
     constexpr int LA = MI * 2 * 16 / 8 / kBigWaves;  // wave-level loads of the A tile per wave per stage
-    constexpr int LB = kBigLB;
+    constexpr int NJe = MI == 8 ? kColumns : kBigNJ;   // block columns the K loop computes (8 outside experiments)
+    constexpr int LB = MI == 8 ? kBigLB - (kBigNJ - NJe) : kBigLB;
     constexpr int NL = LA + LB;                      // loads per wave per K-tile
-    static_assert(NL % 4 == 0, "the loads are queued in four equal portions");
+    static_assert(NL % 4 == 0 || NJe != kBigNJ, "the loads are queued in four equal portions");
     const int wm = (wave >> 1) * (MI * 16), wn = (wave & 1) * 128;
 
     v4f acc[MI][kBigNJ];
@@ -570,13 +576,13 @@ void gemm_nt_big_kernel(const BigLaunch L) {
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
                 // fa[i] is dead after its two MFMAs; it is refilled with the fragment of the next tile one step later
-                acc[i][6] = mfma_16x16x128<FA, FB>(frag(fb[2]), frag(fa[i]), acc[i][6]);
+                acc[i][NJe - 2] = mfma_16x16x128<FA, FB>(frag(fb[(NJe - 2) & 3]), frag(fa[i]), acc[i][NJe - 2]);
                 if (prefetch && !kNoAReads && i > 0) {
                     fa[i - 1][0] = rd_a(s1, i - 1, 0);
                     fa[i - 1][1] = rd_a(s1, i - 1, 1);
                 }
                 sched_fence();
-                acc[i][7] = mfma_16x16x128<FA, FB>(frag(fb[3]), frag(fa[i]), acc[i][7]);
+                acc[i][NJe - 1] = mfma_16x16x128<FA, FB>(frag(fb[(NJe - 1) & 3]), frag(fa[i]), acc[i][NJe - 1]);
                 if constexpr (loads) {   // loads [i kBackLoads / MI, (i + 1) kBackLoads / MI) ride on this step
 #pragma unroll
                     for (int l = i * kBackLoads / MI; l < (i + 1) * kBackLoads / MI; ++l) issue(kt + NS, l);
@@ -624,7 +630,7 @@ void gemm_nt_big_kernel(const BigLaunch L) {
                 sched_fence();
                 int l = 0;
 #pragma unroll
-                for (int j = 0; j < 6; ++j) {
+                for (int j = 0; j < NJe - 2; ++j) {
 #pragma unroll
                     for (int i = 0; i < MI; ++i) {
                         acc[i][j] = mfma_16x16x128<FA, FB>(frag(fb[j & 3]), frag(fa[i]), acc[i][j]);
