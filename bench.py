@@ -933,7 +933,7 @@ def main():
         for lin in mods:   # (only the gate looks at the quantised output gradient)
             lin.keep_quantised_grad, lin.quantised_grad_output = False, None
         graph_note = None
-        if not args.no_graph and not args.weight_stream:
+        if not args.no_graph:
             # two eager steps (the gate's, or these) have given every scaling role its first scale
             for i in range(first, 2):
                 eager_step(i)
