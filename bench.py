@@ -151,6 +151,71 @@ def event_time_ms(fn, reps, warm=3):
     return start.elapsed_time(stop) / reps
 
 
+# ------------------------------------------------------------------------------------ package power
+def _power_files():
+    """(power1_input, power1_cap) of the first GPU's hwmon node, in microwatts; (None, None) where the driver exposes
+    none.  These boxes have one GPU."""
+    import glob
+
+    for d in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
+        f = os.path.join(d, "power1_input")
+        if os.access(f, os.R_OK):
+            cap = os.path.join(d, "power1_cap")
+            return f, cap if os.access(cap, os.R_OK) else None
+    return None, None
+
+
+def package_power(fn, seconds=1.0, period=0.004):
+    """Package power while `fn(i)` is launched back to back for `seconds` (the queue is kept a few calls deep and
+    never drains): a thread reads the driver's power sensor every `period` seconds; the first third of the samples
+    (ramp-up, sensor averaging) is dropped.  Returns None where there is no sensor."""
+    import threading
+
+    import torch
+
+    f, cap = _power_files()
+    if f is None:
+        return None
+    samples, stop = [], threading.Event()
+
+    def sampler():
+        while not stop.is_set():
+            try:
+                samples.append(int(open(f).read()) * 1e-6)
+            except (OSError, ValueError):
+                pass
+            time.sleep(period)
+
+    for i in range(3):
+        fn(i)
+    torch.cuda.synchronize()
+    th = threading.Thread(target=sampler, daemon=True)
+    th.start()
+    t0, i, events = time.perf_counter(), 0, []
+    while time.perf_counter() - t0 < seconds:
+        fn(i)
+        i += 1
+        ev = torch.cuda.Event()
+        ev.record()
+        events.append(ev)
+        if len(events) > 8:
+            events.pop(0).synchronize()
+    torch.cuda.synchronize()
+    stop.set()
+    th.join()
+    kept = samples[len(samples) // 3:]
+    if not kept:
+        return None
+    out = {"watts_mean": round(sum(kept) / len(kept), 1), "watts_max": round(max(kept), 1), "samples": len(kept),
+           "calls": i, "seconds": seconds, "sensor": "hwmon power1_input (package), read every %g ms" % (period * 1e3)}
+    if cap is not None:
+        try:
+            out["cap_watts"] = round(int(open(cap).read()) * 1e-6, 1)
+        except (OSError, ValueError):
+            pass
+    return out
+
+
 # ------------------------------------------------------------------------------------ linear workload
 def build_linears(device, nsets, fp8_out=False):
     """The five linears, and `nsets` steps' worth of inputs resident in HBM: per step and layer a fresh seeded X and
@@ -727,6 +792,25 @@ def loop_experiments(device, reps=3, launches=24):
                 rep = _stamp_report(lib, 256, K // 128)
                 res[name].update({"cycles_per_k_tile": rep["k_loop_cycles_per_k_tile_p50"],
                                   "clock_ghz": rep["k_loop_shader_clock_ghz_p50"]})
+        # package power of every build under the same sustained launches (a pass of its own, about a second each)
+        kp = [0]
+
+        def vpow(i):
+            a, b = views[i % nsets]
+            torch._scaled_mm(a, b.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+
+        pw = package_power(vpow, seconds=0.8)
+        if pw is not None:
+            res[vendor]["watts"] = pw["watts_mean"]
+        for name, lib in libs:
+            def pfn(i, lib=lib):
+                x, w, y = sets[i % nsets]
+                _run_gemms(lib, [(x, w, y, False, False, bf16)], st)
+
+            pw = package_power(pfn, seconds=0.8)
+            if pw is not None:
+                res[name]["watts"] = pw["watts_mean"]
+                out["power_cap_watts"] = pw.get("cap_watts")
         for name in res:
             res[name]["us_best"] = min(res[name]["us"])
             res[name]["tflops"] = round(2.0 * TOKENS * 4096 * K / res[name]["us_best"] / 1e6, 1)
@@ -985,6 +1069,8 @@ def main():
                      "value": round(flops_step / (e_ms * 1e-3) / 1e12, 2)}
         gf, gms, per_call = gemm_in_step_timing(eager_step, first + args.warmup + args.steps, args.steps)
         achieved = gf / (gms * 1e-3) / 1e12
+        # package power while the steps run back to back as in the timed region (a second of them, after everything timed)
+        power = package_power(lambda i: step(first + i), seconds=1.0)
         acts = "e4m3 activations out of the GEMM epilogue" if args.fp8_activations else "bf16 activations"
         out.update({
             "metric": "FP8Linear fwd+bwd TFLOP/s", "value": round(value, 2), "unit": "TFLOP/s", "dtype": "fp8",
@@ -992,6 +1078,7 @@ def main():
                                    "delayed scaling hist 16, fresh seeded X/dY and perturbed weights every step",
                        "weight_requantisation": "second stream, per layer" if args.weight_stream else "compute stream, one batched call per step",
                        "launch": launch, "launch_note": graph_note, "eager_launches": eager,
+                       "package_power_during_steps": power,
                        "tokens": TOKENS, "linears": [f"{n}:{k}->{o}" for n, k, o in LINEARS], "input_sets": len(sets),
                        "flags": flags_of(args), "flops_per_step": flops_step, "pct_fp8_peak": round(100 * value / PEAK_FP8_TFLOPS, 2)},
             "verified": ({"against": "CPU oracle, steps 0 and 1: amax / scales / histories / fp8 bytes bit-exact, "

@@ -40,7 +40,7 @@ __device__ int g_plain_tile_order = 0;
 #define NTFP8_CYCLES(var) var = __builtin_readcyclecounter()
 // Timing experiments on the K loop of whole tiles, chosen when a profiling build is compiled (the results of such a
 // build are wrong, only its stamps mean something).  -DNTFP8_KNOCKOUT=<bits> leaves parts of the loop out: 1 the global
-// loads (stale registers are deposited), 2 the deposits into LDS, 4 the workgroup barrier, 8 the LDS reads of the B
+// loads (the registers of the first K-tile are deposited again and again), 2 the deposits into LDS, 4 the workgroup barrier, 8 the LDS reads of the B
 // fragments, 16 those of the A fragments.  -DNTFP8_IDLE=<n> lets every wave sleep 64 n cycles behind the barrier of
 // every K-tile.  -DNTFP8_COLUMNS=<6 | 7> runs the K loop of a tile that is 192 or 224 columns wide instead of 256 (that
 // many of a wave's eight block columns, B loads and B fragments; the schedule is the same with the last front groups
@@ -609,12 +609,17 @@ void gemm_nt_big_kernel(const BigLaunch L) {
             // than from the memory-side cache stalled the barrier.
             v4i g[NL];
             const int wr_lane = wave * 1024 + lane * 16;   // a wave-level load covers 1 KB of a stage: 16 bytes per lane
+            auto load_now = [&](int ktile, int l) {
+                g[l] = l < LA ? reg_load16(ra, a_off[l], ktile * a_step) : reg_load16(rb, b_off[l - LA], ktile * b_step);
+            };
             if constexpr (kNoLoads) {
+                // one real K-tile, deposited again and again: operand bytes of the real distribution (what the matrix
+                // cores draw depends on the data: zeros would make this build look far cheaper than it is)
 #pragma unroll
-                for (int l = 0; l < NL; ++l) g[l] = (v4i){l, lane, 0, 0};
+                for (int l = 0; l < NL; ++l) load_now(0, l);
             }
             auto request = [&](int ktile, int l) {
-                if constexpr (!kNoLoads) g[l] = l < LA ? reg_load16(ra, a_off[l], ktile * a_step) : reg_load16(rb, b_off[l - LA], ktile * b_step);
+                if constexpr (!kNoLoads) load_now(ktile, l);
             };
             auto deposit = [&](int s, int l) {
                 if constexpr (kNoDeposits) return;
