@@ -811,6 +811,23 @@ def loop_experiments(device, reps=3, launches=24):
             if pw is not None:
                 res[name]["watts"] = pw["watts_mean"]
                 out["power_cap_watts"] = pw.get("cap_watts")
+        # the kernel as it is on all-zero operands: same instructions, same cycles; what the matrix cores draw depends
+        # on the operand bytes, so this shows how fast the schedule runs when power does not hold the clock down
+        base_lib = dict(libs)["base"]
+        zx = FP8Tensor(torch.zeros(TOKENS, K, dtype=torch.bfloat16, device=device), DTypes.FP8E4M3)
+        zw = FP8Tensor(torch.zeros(4096, K, dtype=torch.bfloat16, device=device), DTypes.FP8E4M3)
+        zy = sets[0][2]
+
+        def zfn(i=0):
+            _run_gemms(base_lib, [(zx, zw, zy, False, False, bf16)], st)
+
+        zname = "base_zero_operands"
+        res[zname] = {"us": [round(event_time_ms(zfn, launches, warm=4) * 1e3, 1) for _ in range(reps)]}
+        rep = _stamp_report(base_lib, 256, K // 128)
+        res[zname].update({"cycles_per_k_tile": rep["k_loop_cycles_per_k_tile_p50"], "clock_ghz": rep["k_loop_shader_clock_ghz_p50"]})
+        pw = package_power(zfn, seconds=0.8)
+        if pw is not None:
+            res[zname]["watts"] = pw["watts_mean"]
         for name in res:
             res[name]["us_best"] = min(res[name]["us"])
             res[name]["tflops"] = round(2.0 * TOKENS * 4096 * K / res[name]["us_best"] / 1e6, 1)
