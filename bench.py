@@ -1070,6 +1070,8 @@ def main():
     if args.workload == "linear":
         value = flops_step / (ms_per_step * 1e-3) / 1e12
         launch = "eager" if step is eager_step else "hip graph replay"
+        # package power while the steps run back to back as in the timed region (one more second of them)
+        power = package_power(lambda i: step(first + i), seconds=1.0)
         eager = None
         if step is not eager_step:
             # the same steps launched from Python, for comparison (and the passes the GEMM timing instruments)
@@ -1086,8 +1088,6 @@ def main():
                      "value": round(flops_step / (e_ms * 1e-3) / 1e12, 2)}
         gf, gms, per_call = gemm_in_step_timing(eager_step, first + args.warmup + args.steps, args.steps)
         achieved = gf / (gms * 1e-3) / 1e12
-        # package power while the steps run back to back as in the timed region (a second of them, after everything timed)
-        power = package_power(lambda i: step(first + i), seconds=1.0)
         acts = "e4m3 activations out of the GEMM epilogue" if args.fp8_activations else "bf16 activations"
         out.update({
             "metric": "FP8Linear fwd+bwd TFLOP/s", "value": round(value, 2), "unit": "TFLOP/s", "dtype": "fp8",
