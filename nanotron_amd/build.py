@@ -42,6 +42,7 @@ EXPERIMENTS = {
     "mfma_only": ["-DNTFP8_KNOCKOUT=31"],
     "idle_256": ["-DNTFP8_IDLE=4"],
     "idle_512": ["-DNTFP8_IDLE=8"],
+    "mfma_only_32x32x64": ["-DNTFP8_KNOCKOUT=31", "-DNTFP8_MFMA32=1"],
     "columns_224": ["-DNTFP8_COLUMNS=7"],
     "columns_192": ["-DNTFP8_COLUMNS=6"],
 }

@@ -45,6 +45,9 @@ __device__ int g_plain_tile_order = 0;
 // every K-tile.  -DNTFP8_COLUMNS=<6 | 7> runs the K loop of a tile that is 192 or 224 columns wide instead of 256 (that
 // many of a wave's eight block columns, B loads and B fragments; the schedule is the same with the last front groups
 // left out): what a tile width that divides N = 6144 or 14336 into a whole number of rounds would cost per K-tile.
+// -DNTFP8_MFMA32=1 (with -DNTFP8_KNOCKOUT=31) issues 32 V_MFMA_F32_32X32X64_F8F6F4 per K-tile in place of the 64
+// 16x16x128 ones (the same FLOPs and matrix-pipe cycles, half the operand registers read per FLOP, twice the accumulator
+// registers touched): what the other instruction shape draws.
 #ifndef NTFP8_KNOCKOUT
 #define NTFP8_KNOCKOUT 0
 #endif
@@ -54,11 +57,16 @@ __device__ int g_plain_tile_order = 0;
 #ifndef NTFP8_COLUMNS
 #define NTFP8_COLUMNS 8
 #endif
+#ifndef NTFP8_MFMA32
+#define NTFP8_MFMA32 0
+#endif
 constexpr int kKnockout = NTFP8_KNOCKOUT, kIdle = NTFP8_IDLE, kColumns = NTFP8_COLUMNS;
+constexpr bool kMfma32 = NTFP8_MFMA32 != 0;
 #else
 #define NTFP8_STAMP(var) (void)0
 #define NTFP8_CYCLES(var) (void)0
 constexpr int kKnockout = 0, kIdle = 0, kColumns = 8;
+constexpr bool kMfma32 = false;
 #endif
 constexpr bool kNoLoads = kKnockout & 1, kNoDeposits = kKnockout & 2, kNoBarrier = kKnockout & 4, kNoBReads = kKnockout & 8,
                kNoAReads = kKnockout & 16;
@@ -401,6 +409,28 @@ void gemm_nt_big_kernel(const BigLaunch L) {
     for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < kBigNJ; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    // (experiment builds only: the accumulators of the 32 x 32 instruction shape)
+    [[maybe_unused]] v16f big[kMfma32 ? MI / 2 : 1][kMfma32 ? kBigNJ / 2 : 1];
+    if constexpr (kMfma32) {
+#pragma unroll
+        for (int i = 0; i < MI / 2; ++i)
+#pragma unroll
+            for (int j = 0; j < kBigNJ / 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) big[i][j][e] = 0.f;
+    }
+    // one step of the MFMA loop: block (i, j) of the wave tile; in the 32 x 32 experiment every fourth step issues the
+    // two instructions (K = 2 x 64) of the 32 x 32 block it belongs to, on whatever fragments are at hand
+    auto mma = [&](int i, int j, const v8i b, const v8i a) {
+        if constexpr (kMfma32) {
+            if (!(i & 1) && !(j & 1)) {
+                big[i >> 1][j >> 1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b, a, big[i >> 1][j >> 1], FB, FA, 0, 0, 0, 0);
+                big[i >> 1][j >> 1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, big[i >> 1][j >> 1], FB, FA, 0, 0, 0, 0);
+            }
+        } else {
+            acc[i][j] = mfma_16x16x128<FA, FB>(b, a, acc[i][j]);
+        }
+    };
 
     // The K loop.  kAT: the A operand is given as its transpose, a [K, M] tensor (what wgrad has of dY: its reduction
     // index, the token, is the row index).  Its K-tiles lie in LDS as they lie in memory, 128 rows of k with 256 (whole
@@ -551,7 +581,7 @@ void gemm_nt_big_kernel(const BigLaunch L) {
                 const int lend = (loads && j < 2) ? l + kFrontLoads / 2 : l;
 #pragma unroll
                 for (int i = 0; i < MI; ++i) {
-                    acc[i][j] = mfma_16x16x128<FA, FB>(frag(fb[j & 3]), frag(fa[i]), acc[i][j]);
+                    mma(i, j, frag(fb[j & 3]), frag(fa[i]));
                     if (i == 0) fb[(j + 2) & 3][0] = rd_b(s, j + 2, 0);
                     else if (i == 2) fb[(j + 2) & 3][1] = rd_b(s, j + 2, 1);
                     else if (l < lend) issue(kt + NS - 1, l++);
@@ -576,13 +606,13 @@ void gemm_nt_big_kernel(const BigLaunch L) {
 #pragma unroll
             for (int i = 0; i < MI; ++i) {
                 // fa[i] is dead after its two MFMAs; it is refilled with the fragment of the next tile one step later
-                acc[i][NJe - 2] = mfma_16x16x128<FA, FB>(frag(fb[(NJe - 2) & 3]), frag(fa[i]), acc[i][NJe - 2]);
+                mma(i, NJe - 2, frag(fb[(NJe - 2) & 3]), frag(fa[i]));
                 if (prefetch && !kNoAReads && i > 0) {
                     fa[i - 1][0] = rd_a(s1, i - 1, 0);
                     fa[i - 1][1] = rd_a(s1, i - 1, 1);
                 }
                 sched_fence();
-                acc[i][NJe - 1] = mfma_16x16x128<FA, FB>(frag(fb[(NJe - 1) & 3]), frag(fa[i]), acc[i][NJe - 1]);
+                mma(i, NJe - 1, frag(fb[(NJe - 1) & 3]), frag(fa[i]));
                 if constexpr (loads) {   // loads [i kBackLoads / MI, (i + 1) kBackLoads / MI) ride on this step
 #pragma unroll
                     for (int l = i * kBackLoads / MI; l < (i + 1) * kBackLoads / MI; ++l) issue(kt + NS, l);
@@ -638,7 +668,7 @@ void gemm_nt_big_kernel(const BigLaunch L) {
                 for (int j = 0; j < NJe - 2; ++j) {
 #pragma unroll
                     for (int i = 0; i < MI; ++i) {
-                        acc[i][j] = mfma_16x16x128<FA, FB>(frag(fb[j & 3]), frag(fa[i]), acc[i][j]);
+                        mma(i, j, frag(fb[j & 3]), frag(fa[i]));
                         if (i == 0) { if constexpr (!kNoBReads) fb[(j + 2) & 3][0] = rd_b(s, j + 2, 0); }
                         else if (i == 2) { if constexpr (!kNoBReads) fb[(j + 2) & 3][1] = rd_b(s, j + 2, 1); }
                         else if (l < NL) {
@@ -762,6 +792,14 @@ void gemm_nt_big_kernel(const BigLaunch L) {
 
     NTFP8_STAMP(st_loop);
     NTFP8_CYCLES(cy_loop);
+    if constexpr (kMfma32) {   // the experiment's results must reach memory, or its MFMAs are dead code
+#pragma unroll
+        for (int i = 0; i < MI / 2; ++i)
+#pragma unroll
+            for (int j = 0; j < kBigNJ / 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[2 * i + (e >> 3)][2 * j + ((e >> 2) & 1)][e & 3] += big[i][j][e];
+    }
     {
         // output type, accumulation and bias are properties of the problem, not of the kernel (fp8 outputs apart)
         auto epilogue = [&](auto bias_tag, const float (*bv)[4]) {
