@@ -327,8 +327,9 @@ def gemm_in_step_timing(step, first_index, steps):
     def timed_one(a, b, out_dtype, accumulate_into, bias=None):
         return bracket(lambda: orig_one(a, b, out_dtype, accumulate_into, bias), [(a.shape[0], b.shape[0], a.shape[1])])
 
-    def timed_fp8(a, b, dtype, state, with_transpose, bias=None):
-        return bracket(lambda: orig_fp8(a, b, dtype, state, with_transpose, bias), [(a.shape[0], b.shape[0], a.shape[1])])
+    def timed_fp8(a, b, dtype, state, with_transpose, bias=None, bt=False, at=False):
+        mnk = (a.shape[1 if at else 0], b.shape[1 if bt else 0], a.shape[0 if at else 1])
+        return bracket(lambda: orig_fp8(a, b, dtype, state, with_transpose, bias, bt, at), [mnk])
 
     def timed_batch(problems):
         # elements 5 and 7 of a problem mark operands handed over as their transposes ([K, N] / [K, M])
