@@ -304,6 +304,66 @@ def test_gradient_of_an_fp8_activation_goes_back_as_fp8_bytes():
     assert second.fp8_grad_inputs_sent == sent[0] + 1
 
 
+def test_fp8_activation_and_gradient_between_the_benchmark_mlp_linears_at_full_size():
+    """The fp8 hand-over in both directions at the benchmark's size: up projection 4096 -> 14336 with an e4m3 output,
+    down projection 14336 -> 4096, 4096 tokens, bf16 master weights, three delayed-scaling steps.  Forward: the bytes of
+    the activation equal the delayed-scaling quantisation of the fp32 result of the same GEMM.  Backward: the e5m2 bytes
+    the down projection's dgrad epilogue leaves for the up projection (896 whole tiles and a half-tile tail, operands
+    read untransposed) equal the quantisation of its fp32 dgrad result under the same role; the up projection's own
+    gradients are compared with the oracle on sampled rows."""
+    from nanotron_amd.fp8 import DTypes, FP8Linear, FP8Parameter, FP8Tensor
+    from nanotron_amd.fp8.kernel import fp8_matmul_kernel
+
+    T, H, I = 4096, 4096, 14336
+    g = torch.Generator(device="cuda").manual_seed(11)
+    up = FP8Linear(H, I, bias=False, device="cuda", dtype=torch.bfloat16, out_dtype=DTypes.FP8E4M3, delayed_scaling=True)
+    down = FP8Linear(I, H, bias=False, device="cuda", dtype=torch.bfloat16, out_dtype=torch.bfloat16, delayed_scaling=True)
+    up.weight = FP8Parameter((torch.randn(I, H, generator=g, device="cuda") * 0.02).to(torch.bfloat16), DTypes.FP8E4M3)
+    down.weight = FP8Parameter((torch.randn(H, I, generator=g, device="cuda") * 0.02).to(torch.bfloat16), DTypes.FP8E4M3)
+    up.keep_quantised_grad = down.keep_quantised_grad = True
+    rows = torch.arange(0, T, 67, device="cuda")[:48]
+    sent = 0
+    for step in range(3):
+        x = (torch.randn(T, H, generator=g, device="cuda") * (1.0 + 0.5 * step)).to(torch.bfloat16).requires_grad_(True)
+        gy = (torch.randn(T, H, generator=g, device="cuda") * 1e-3 * (1 + step)).to(torch.bfloat16)
+        out_role, grad_role = up.scaling["output"], up.scaling["output_grad"]
+        bwd_fused = grad_role.initialised
+        out_before, grad_before = _clone_state(out_role), _clone_state(grad_role)
+        h = up(x)
+        assert isinstance(h, FP8Tensor) and tuple(h.shape) == (T, I)
+        # forward: the activation against the long way on the operands the layer used (a role without a scale yet
+        # quantises with current scaling either way)
+        xq = h._grad_handle.grad_fn.saved_tensors[0]
+        r32 = fp8_matmul_kernel(mat_a=up.weight.data, transpose_a=True, mat_b=xq, transpose_b=False, use_split_accumulator=False)
+        want_h = FP8Tensor(r32, DTypes.FP8E4M3, state=out_before)
+        assert torch.equal(h.as_subclass(torch.Tensor), want_h.as_subclass(torch.Tensor)), step
+        assert _same_f32(h.fp8_meta.scale, want_h.fp8_meta.scale) and _same_f32(out_role._buf, out_before._buf), step
+        del r32, want_h
+        y = down(h)
+        y.backward(gy)
+        dx32 = fp8_matmul_kernel(mat_a=down.weight.data, transpose_a=False, mat_b=down.quantised_grad_output,
+                                 transpose_b=False, use_split_accumulator=True)
+        got = up.quantised_grad_output
+        assert isinstance(got, FP8Tensor) and got.fp8_meta.dtype == DTypes.FP8E5M2 and tuple(got.shape) == (T, I)
+        if bwd_fused:
+            sent += 1
+            assert down.fp8_grad_inputs_sent == sent
+            want = FP8Tensor(dx32, DTypes.FP8E5M2, state=grad_before)
+            assert torch.equal(got.as_subclass(torch.Tensor), want.as_subclass(torch.Tensor)), step
+            assert _same_f32(got.fp8_meta.scale, want.fp8_meta.scale) and _same_f32(got.fp8_meta.amax, want.fp8_meta.amax), step
+            assert _same_f32(grad_role._buf, grad_before._buf), step
+        else:
+            want = FP8Tensor(dx32.to(h._grad_handle.dtype), DTypes.FP8E5M2, state=grad_before)
+            assert torch.equal(got.as_subclass(torch.Tensor), want.as_subclass(torch.Tensor)), step
+        # the up projection's gradients from those bytes, against the oracle on sampled rows of dX and of dW
+        gq = O.Quantised(got.as_subclass(torch.Tensor)[rows].cpu(), got.fp8_meta.amax.cpu(), got.fp8_meta.scale.cpu(), O.E5M2)
+        wq = O.Quantised(up.weight.data.as_subclass(torch.Tensor).cpu(), up.weight.data.fp8_meta.amax.cpu(),
+                         up.weight.data.fp8_meta.scale.cpu(), O.E4M3)
+        assert O.rel_l2(x.grad[rows].float().cpu(), O.linear_dgrad(gq, wq, torch.bfloat16).float()) <= 1e-3, step
+        assert up.weight.main_grad is not None and bool(torch.isfinite(up.weight.main_grad).all())
+    assert sent >= 1
+
+
 def test_an_fp8_activation_that_lost_its_gradient_handle_is_refused():
     """The gradient of an fp8 activation travels through the `_grad_handle` attribute of the object the producing layer
     returned.  A tensor derived from it (here: the same bytes re-wrapped, meta carried over) has no handle; consuming it
