@@ -544,6 +544,16 @@ def stream_probe_ms(bufs, reps):
                      "ntfp8_stream_probe")
 
         res[name] = event_time_ms(fn, reps, warm=8)
+    # the same copy by the vendor's kernel (torch's copy_ of a contiguous tensor), for scale
+    views = [b.view(torch.uint8).reshape(-1) for b in bufs]
+    k = [0]
+
+    def vcopy():
+        i = k[0]
+        k[0] += 1
+        dst[i % 2].copy_(views[i % len(views)])
+
+    res["copy_by_torch"] = event_time_ms(vcopy, reps, warm=8)
     return res
 
 
@@ -572,9 +582,9 @@ def quant_report(device, traffic):
                         "algorithmic_bytes": qb, "kernel": "quant_flat_kernel",
                         "frac_of_yardstick": round(probe["read_2B_write_1B"] / q_avg, 4)},
            "yardstick": {"what": "ntfp8_stream_probe on the same tensors: same grid and 128-bit streaming accesses, no arithmetic, "
-                                 "no reduction",
+                                 "no reduction; copy_by_torch: the same copy by torch's copy_",
                          **{k: {"ms": round(v, 5), "GBps": round(b * 4096 * 4096 / (v * 1e-3) / 1e9, 1)}
-                            for (k, v), b in zip(probe.items(), (2.0, 3.0, 4.0))}},
+                            for (k, v), b in zip(probe.items(), (2.0, 3.0, 4.0, 4.0))}},
            "both_formats_one_pass": {"ms": round(dual_ms, 5), "algorithmic_bytes": 4.0 * 4096 * 4096,
                                      "GBps": round(4.0 * 4096 * 4096 / (dual_ms * 1e-3) / 1e9, 1),
                                      "frac": round(4.0 * 4096 * 4096 / (dual_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
@@ -595,6 +605,8 @@ def quant_report(device, traffic):
                                             "frac": round(nbytes / (avg * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
                                             "yardstick_read_2B_write_1B_ms": round(pr["read_2B_write_1B"], 5),
                                             "yardstick_read_only_GBps": round(2.0 * shape[0] * shape[1] / (pr["read_only"] * 1e-3) / 1e9, 1),
+                                            "yardstick_copy_GBps": round(4.0 * shape[0] * shape[1] / (pr["copy"] * 1e-3) / 1e9, 1),
+                                            "copy_by_torch_GBps": round(4.0 * shape[0] * shape[1] / (pr["copy_by_torch"] * 1e-3) / 1e9, 1),
                                             "frac_of_yardstick": round(pr["read_2B_write_1B"] / avg, 4)}
         del lb
     rep["large_tensors"] = large
@@ -1137,9 +1149,9 @@ def main():
         yard = stream_probe_ms(bufs, 64)
         out["roofline"]["frac_of_yardstick"] = round(yard["read_2B_write_1B"] / q_avg, 4)
         out["yardstick"] = {"what": "ntfp8_stream_probe on the same tensors: same grid and 128-bit streaming accesses, no arithmetic, "
-                                    "no reduction",
+                                    "no reduction; copy_by_torch: the same copy by torch's copy_",
                             **{k: {"ms": round(v, 5), "GBps": round(b * 4096 * 4096 / (v * 1e-3) / 1e9, 1)}
-                               for (k, v), b in zip(yard.items(), (2.0, 3.0, 4.0))}}
+                               for (k, v), b in zip(yard.items(), (2.0, 3.0, 4.0, 4.0))}}
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_baseline_quant()
     print(json.dumps(out))
